@@ -768,6 +768,49 @@ int semipd_probe_cu_placement(int32_t* out, int num_workgroups, int64_t spin_cyc
  * events it uses around a hot kernel to calibrate the dispatch + completion overhead the pair adds. */
 int semipd_launch_noop(int count, void* stream);
 
+/* ------------------------------------------------------------------ */
+/* block-local attention with a sink term                              */
+/* ------------------------------------------------------------------ */
+/* The step between a projection GEMM and the attention below, one launch.  Row t of qkv (row stride ld elements)
+ * holds q | k | v at columns 0, k_off, v_off.  Per head: q <- q / sqrt(mean(q^2) + eps) in place; the same for k,
+ * written to k_pool[loc[t]]; v, or (1 - a) v + a v_first[t] when v_first is given (a = the one element `mix` points to,
+ * on the device), written to v_pool[loc[t]].  Sums, division and blend in fp32.  Pools are [N, kv heads, size] of the
+ * activation type.  No reference counterpart. */
+int semipd_unit_norm_kv_store(void* qkv, int64_t ld, int64_t num_tokens, int num_q_heads, int num_kv_heads, int qk_dim,
+                              int v_dim, int64_t k_off, int64_t v_off, float eps, const void* v_first, int64_t v_first_ld,
+                              const void* mix, void* k_pool, void* v_pool, const int64_t* loc, int dtype, void* stream);
+/* Attention of prompt portions and decode steps over the paged pools, keys found through the request's row of
+ * req_to_token: a query at position p of its sequence sees keys lo(p) .. p with lo(p) = floor(p / chunk) * chunk
+ * (chunk 0: every earlier key).  score = cap * tanh(scale * q.k / cap) (cap 0: scale * q.k); the softmax denominator
+ * also holds exp(sink[head]) (sink NULL: none), a term without a value row.  out = softmax . V, times sigmoid(gate)
+ * where gate is given.  Request b's queries are rows q_start[b] .. + q_len[b] and end at position seq_lens[b] - 1; with
+ * q_start == NULL row b is request b's newest token.  max_q_len: the largest q_len (host value, sizes the grid).
+ * form: 0 = chosen by shape and type, 1 = one wave per row (every type and size), 2 = matrix-core forms (bf16 / f16,
+ * qk_dim % 32 == 0, v_dim % 16 == 0).  Scores, softmax and accumulation in fp32.  No reference counterpart. */
+int semipd_local_attention(const void* q, int64_t q_ld, const void* gate, int64_t gate_ld, void* out, int64_t out_ld,
+                           const void* k_pool, const void* v_pool, const int32_t* req_to_token,
+                           int64_t req_to_token_stride, const int64_t* req_pool_indices, const int64_t* seq_lens,
+                           const int32_t* q_start, const int32_t* q_len, int64_t batch, int64_t num_tokens,
+                           int64_t max_q_len, int num_q_heads, int num_kv_heads, int qk_dim, int v_dim, const float* sink,
+                           float scale, float logit_cap, int chunk, int form, int dtype, void* stream);
+/* 1 when form 2 of semipd_local_attention takes these sizes and this type. */
+int semipd_local_attention_mfma_supported(int num_q_heads, int num_kv_heads, int qk_dim, int v_dim, int dtype);
+
+/* ------------------------------------------------------------------ */
+/* LayerNorm of post-norm residual blocks, squared ReLU                */
+/* ------------------------------------------------------------------ */
+/* Per row: y = (x + in_bias - mean) / sqrt(var + eps) * weight + bias, var = mean of the squared deviations, fp32
+ * arithmetic; x rows are fp32 (in_is_f32) or of `dtype`, in_bias (may be NULL), weight and bias of `dtype`.  With
+ * `residual` (fp32 rows, updated in place) y is added to it and the sum is what `out` (rows of `dtype`, may be NULL
+ * then) receives: "stream += norm(sublayer output)" plus the next GEMM's input in one launch.  Strides in elements.
+ * No reference counterpart. */
+int semipd_layernorm(const void* in, int64_t in_ld, int in_is_f32, const void* in_bias, const void* weight,
+                     const void* bias, float eps, float* residual, int64_t residual_ld, void* out, int64_t out_ld,
+                     int64_t rows, int64_t width, int dtype, void* stream);
+/* u <- max(u + bias, 0)^2 in place, rows of `width` elements with stride ld; bias may be NULL.  No reference
+ * counterpart. */
+int semipd_bias_relu_square(void* u, int64_t ld, const void* bias, int64_t rows, int64_t width, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -147,6 +147,12 @@ _SIGNATURES = {
     "semipd_ep_dispatch": [_vp, _vp, _vp, _vp, _i64, _i32, _i64, _i32, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp],
     "semipd_ep_combine": [_vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i32, _i64, _i32, _i32, _vp],
     "semipd_ar_dispose": [_vp],
+    "semipd_layernorm": [_vp, _i64, _i32, _vp, _vp, _vp, _f32, _vp, _i64, _vp, _i64, _i64, _i64, _i32, _vp],
+    "semipd_bias_relu_square": [_vp, _i64, _vp, _i64, _i64, _i32, _vp],
+    "semipd_unit_norm_kv_store": [_vp, _i64, _i64, _i32, _i32, _i32, _i32, _i64, _i64, _f32, _vp, _i64, _vp, _vp, _vp, _vp, _i32, _vp],
+    "semipd_local_attention": [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32,
+                               _i32, _i32, _vp, _f32, _f32, _i32, _i32, _i32, _vp],
+    "semipd_local_attention_mfma_supported": [_i32, _i32, _i32, _i32, _i32],
 }
 _RESTYPES = {"semipd_last_error": C.c_char_p, "semipd_lm_head_argmax_workspace": _sz,
              "semipd_linear_workspace": _sz, "semipd_stream_linear_workspace": _sz, "semipd_dense_gemm_report": _sz, "semipd_ar_meta_size": _sz, "semipd_ar_region_size": _sz}

@@ -197,6 +197,8 @@ class HipAttnBackend(AttentionBackend):
         geo = self.model_runner.kv_geometry
         if geo["kind"] == "mla":
             return geo["kv_lora_rank"] + geo["qk_rope_head_dim"]  # K and V share the latent row
+        if isinstance(geo["head_dim"], (list, tuple)):      # layers of their own geometry: the widest row (accounting only)
+            return max(d + dv for d, dv in zip(geo["head_dim"], geo["v_head_dim"]))
         return geo["head_dim"] + geo["v_head_dim"]
 
     def _timing(self):
@@ -243,6 +245,31 @@ class HipAttnBackend(AttentionBackend):
             kt.stop("decode_attention", t0, *self._algo, n_kernels=2 if md.num_kv_splits > 1 else 1)
         return o
 
+
+    # ---- block-local attention with a sink term: prompt portions and decode steps over the pools -------------------
+    def forward_local(self, q, layer, forward_batch: ForwardBatch, gate=None):
+        """Attention for layers whose keys and values are in the pool already (the model stored them with the step that
+        prepares q): q [T, heads * head_dim] (may be a column range), keys found through req_to_token, so an extend batch
+        -- whole prompts, portions with a cached prefix, single tokens of running requests side by side -- and a decode
+        batch are the same call.  Mask, cap and sink come from the layer descriptor; `gate` multiplies sigmoid(gate) in."""
+        T = q.shape[0]
+        o = torch.empty((T, layer.tp_q_head_num * layer.v_head_dim), dtype=q.dtype, device=q.device)
+        pool = forward_batch.token_to_kv_pool
+        if forward_batch.forward_mode.is_decode():
+            q_start = q_len = None
+            max_q = 1
+        else:
+            q_start, q_len = forward_batch.extend_start_loc, forward_batch.extend_seq_lens
+            max_q = max(forward_batch.extend_seq_lens_cpu)
+        kt = self._timing()
+        t0 = kt.start() if kt else None
+        ops.local_attention_fwd(q, o, pool.get_key_buffer(layer.layer_id), pool.get_value_buffer(layer.layer_id),
+                                self.req_to_token, forward_batch.req_pool_indices, forward_batch.seq_lens, q_start, q_len, max_q,
+                                layer.scaling, layer.logit_cap, layer.chunk_size, layer.sink, gate,
+                                form=int(os.environ.get("SEMIPD_LOCAL_ATTN_FORM", "0")))
+        if kt:
+            kt.stop("decode_attention" if forward_batch.forward_mode.is_decode() else "extend_attention", t0, 0.0, 0.0)
+        return o
 
     # ---- decode: RoPE + KV store + attention + split merge in one launch -------------------------
     def fused_decode_waves(self, bs: int, head_dim: int, num_kv_splits: int = 0) -> int:
@@ -309,7 +336,7 @@ class RadixAttention:
     layer id; forward() reshapes nothing and dispatches to the batch's backend."""
 
     def __init__(self, num_heads: int, head_dim: int, scaling: float, num_kv_heads: int, layer_id: int,
-                 logit_cap: float = 0.0, v_head_dim: int = -1):
+                 logit_cap: float = 0.0, v_head_dim: int = -1, chunk_size: int = 0, sink: Optional[torch.Tensor] = None):
         self.tp_q_head_num = num_heads
         self.tp_k_head_num = num_kv_heads
         self.tp_v_head_num = num_kv_heads
@@ -319,6 +346,11 @@ class RadixAttention:
         self.scaling = scaling
         self.layer_id = layer_id
         self.logit_cap = logit_cap
+        # block-local attention (HipAttnBackend.forward_local): a query sees the keys of its own block of chunk_size positions,
+        # counted from the start of the sequence (0: all earlier keys); sink: fp32 [heads], one more term exp(sink) in each
+        # head's softmax denominator
+        self.chunk_size = int(chunk_size)
+        self.sink = sink
 
     def forward(self, q, k, v, forward_batch: ForwardBatch, save_kv_cache: bool = True):
         return forward_batch.attn_backend.forward(q, k, v, self, forward_batch, save_kv_cache)

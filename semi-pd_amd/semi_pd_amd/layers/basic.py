@@ -52,6 +52,24 @@ class RMSNorm(nn.Module):
         return x, residual, x_quant
 
 
+class LayerNorm(nn.Module):
+    """LayerNorm with weight and bias on the HIP kernel (csrc/layernorm.hip): mean, biased variance, division and affine
+    map in fp32 whatever the activation type.  forward_add is the post-norm residual block's tail: the fp32 stream takes
+    `+= norm(y)` in place and comes back in the activation type for the next GEMM."""
+
+    def __init__(self, hidden_size: int, eps: float = 1e-5, dtype=None):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(hidden_size, dtype=dtype), requires_grad=False)
+        self.bias = nn.Parameter(torch.zeros(hidden_size, dtype=dtype), requires_grad=False)
+        self.eps = eps
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.layernorm(x, self.weight, self.bias, self.eps)
+
+    def forward_add(self, y: torch.Tensor, residual: torch.Tensor, in_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return ops.layernorm(y, self.weight, self.bias, self.eps, residual=residual, in_bias=in_bias)
+
+
 class SiluAndMul(nn.Module):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return ops.silu_and_mul(x)
@@ -612,7 +630,11 @@ class LogitsProcessor(nn.Module):
 
     def forward(self, input_ids, hidden_states: torch.Tensor, lm_head: VocabParallelEmbedding,
                 forward_batch) -> LogitsProcessorOutput:
-        if forward_batch.forward_mode.is_extend():
+        if forward_batch.forward_mode.is_extend() and getattr(forward_batch, "extend_logit_rows", None) is not None:
+            # logits of chosen prompt positions instead of each request's last one (rows of the flat token axis): scoring
+            # given text, replaying a trace (the role of logprob_start_len, logits_processor.py:232-300)
+            pruned = ops.gather_rows(hidden_states, forward_batch.extend_logit_rows)
+        elif forward_batch.forward_mode.is_extend():
             last_index = torch.cumsum(forward_batch.extend_seq_lens, dim=0, dtype=torch.int64) - 1
             pruned = ops.gather_rows(hidden_states, last_index)
         else:
@@ -621,7 +643,7 @@ class LogitsProcessor(nn.Module):
         # library GEMM + argmax takes 0.36 (profiles/r02_kbench_all_final_tree.txt), at <= 64 rows it is at par or ahead
         # and returns fp32 logits.  Above that the reference's own form: bf16 GEMM, then fp32 (logits_processor.py:394-445).
         if get_tensor_model_parallel_world_size() == 1 and self.final_logit_softcapping is None \
-                and pruned.shape[0] <= LM_HEAD_FUSED_MAX_ROWS:
+                and pruned.shape[0] <= LM_HEAD_FUSED_MAX_ROWS and pruned.dtype in (torch.bfloat16, torch.float16):
             # rows >= vocab_size are padding (vocab_parallel_embedding.py pads to a multiple of 64)
             logits, ids = ops.lm_head_argmax(pruned.contiguous(), lm_head.weight[: self.vocab_size],
                                              return_logits=True)

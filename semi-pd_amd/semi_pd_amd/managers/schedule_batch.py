@@ -102,6 +102,16 @@ class ChunkCache:
         kv_indices = self.req_to_token_pool.req_to_token[req.req_pool_idx, : len(req.fill_ids)]
         req.prefix_indices = kv_indices.to(torch.int64).clone()
 
+    def release_req(self, req: Req):
+        """Give back everything a request holds -- its row of req_to_token and the slot of EVERY token in kv_slots -- for
+        requests that end where their input ends (nothing sampled, so no token without a slot)."""
+        if req.req_pool_idx is not None:
+            self.req_to_token_pool.free(req.req_pool_idx)
+            req.req_pool_idx = None
+        self.token_to_kv_pool_allocator.free(req.kv_slots)
+        req.kv_slots = []
+        req.prefix_indices = torch.empty(0, dtype=torch.int64)
+
     def evictable_size(self):
         return 0
 
@@ -120,6 +130,7 @@ class ModelWorkerBatch:
     sampling_info: Optional[SamplingBatchInfo] = None
     return_logprob: bool = False
     top_logprobs_nums: Optional[List[int]] = None
+    extend_logit_rows: Optional[torch.Tensor] = None   # see ForwardBatch.extend_logit_rows
 
 
 def host_list_to_device(values, dtype, device) -> torch.Tensor:
@@ -308,7 +319,8 @@ class ScheduleBatch:
             extend_prefix_lens=self.prefix_lens if ext else None,
             sampling_info=SamplingBatchInfo.from_reqs(self.reqs, getattr(self, "vocab_size", 0), self.device),
             return_logprob=any(r.return_logprob for r in self.reqs),
-            top_logprobs_nums=[r.top_logprobs_num if r.return_logprob else 0 for r in self.reqs])
+            top_logprobs_nums=[r.top_logprobs_num if r.return_logprob else 0 for r in self.reqs],
+            extend_logit_rows=getattr(self, "extend_logit_rows", None) if ext else None)
 
 
 class AddReqResult(Enum):

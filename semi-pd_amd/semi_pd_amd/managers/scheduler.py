@@ -40,6 +40,11 @@ class TpModelWorker:
         next_token_ids = self.model_runner.sample(logits_output, forward_batch)
         return logits_output, next_token_ids
 
+    def forward_batch_logits(self, model_worker_batch):
+        """The same forward without the sampler: for callers that bring the tokens themselves (managers/replay_scheduler.py)."""
+        forward_batch = ForwardBatch.init_new(model_worker_batch, self.model_runner)
+        return self.model_runner.forward(forward_batch)
+
 
 class SchedulerBase:
     """State and helpers shared by the unified, prefill and decode schedulers."""

@@ -162,27 +162,64 @@ def ipc_safe_zeros(shape, dtype: torch.dtype, device) -> torch.Tensor:
 
 
 class MHATokenToKVPool:
-    def __init__(self, size: int, page_size: int, dtype: torch.dtype, head_num: int, head_dim: int,
-                 layer_num: int, device: str, bypass_create_buffers: bool = False):
+    """K and V rows of every layer.  Layers of one geometry whose values are as wide as their keys share the slab
+    kv[L, 2, N + page, Hkv, D] of the module docstring.  `head_num` / `head_dim` / `v_head_dim` may also be given per layer
+    (lists of layer_num entries) or with values narrower or wider than keys: the rows then live in ONE byte slab, layer
+    after layer, keys [N + page, Hkv_l, D_l] in front of values [N + page, Hkv_l, Dv_l], each region starting on a
+    256-byte boundary -- still one allocation and one IPC handle."""
+
+    def __init__(self, size: int, page_size: int, dtype: torch.dtype, head_num, head_dim,
+                 layer_num: int, device: str, bypass_create_buffers: bool = False, v_head_dim=None):
         assert page_size == 1, "Semi-PD runs with token-granular pages (schedule_batch.py:937)"
         self.size, self.page_size, self.dtype = size, page_size, dtype
-        self.head_num, self.head_dim, self.layer_num, self.device = head_num, head_dim, layer_num, device
+        self.layer_num, self.device = layer_num, device
+
+        def per_layer(x):
+            return [int(v) for v in x] if isinstance(x, (list, tuple)) else [int(x)] * layer_num
+
+        self.head_nums, self.head_dims = per_layer(head_num), per_layer(head_dim)
+        self.v_head_dims = per_layer(v_head_dim) if v_head_dim is not None else list(self.head_dims)
+        assert len(self.head_nums) == len(self.head_dims) == len(self.v_head_dims) == layer_num
+        self.uniform = (len(set(self.head_nums)) == 1 and len(set(self.head_dims)) == 1
+                        and self.v_head_dims == self.head_dims)
+        self.head_num, self.head_dim = self.head_nums[0], self.head_dims[0]
         self.k_buffer: List[torch.Tensor] = []
         self.v_buffer: List[torch.Tensor] = []
         self.slab: Optional[torch.Tensor] = None
         if not bypass_create_buffers:
             self._create_buffers()
 
+    def _regions(self):
+        """(key offset, value offset) in bytes of every layer inside the byte slab, and the slab's size."""
+        rows, es, off, out = self.size + self.page_size, self.dtype.itemsize, 0, []
+        for h, d, dv in zip(self.head_nums, self.head_dims, self.v_head_dims):
+            k_off = off
+            off = -(-(off + rows * h * d * es) // 256) * 256
+            v_off = off
+            off = -(-(off + rows * h * dv * es) // 256) * 256
+            out.append((k_off, v_off))
+        return out, off
+
     def _create_buffers(self):
-        # [L, 2, N+page, Hkv, D]: one allocation, one IPC handle
-        self.slab = ipc_safe_zeros((self.layer_num, 2, self.size + self.page_size, self.head_num, self.head_dim),
-                                   self.dtype, self.device)
-        self.k_buffer = [self.slab[i, 0] for i in range(self.layer_num)]
-        self.v_buffer = [self.slab[i, 1] for i in range(self.layer_num)]
+        if self.uniform:
+            # [L, 2, N+page, Hkv, D]: one allocation, one IPC handle
+            self.slab = ipc_safe_zeros((self.layer_num, 2, self.size + self.page_size, self.head_num, self.head_dim),
+                                       self.dtype, self.device)
+            self.k_buffer = [self.slab[i, 0] for i in range(self.layer_num)]
+            self.v_buffer = [self.slab[i, 1] for i in range(self.layer_num)]
+            return
+        regions, total = self._regions()
+        self.slab = ipc_safe_zeros((total,), torch.uint8, self.device)
+        rows, es = self.size + self.page_size, self.dtype.itemsize
+        for (k_off, v_off), h, d, dv in zip(regions, self.head_nums, self.head_dims, self.v_head_dims):
+            self.k_buffer.append(self.slab[k_off: k_off + rows * h * d * es].view(self.dtype).view(rows, h, d))
+            self.v_buffer.append(self.slab[v_off: v_off + rows * h * dv * es].view(self.dtype).view(rows, h, dv))
 
     def get_kv_size_bytes(self):
-        n = (self.size + self.page_size) * self.head_num * self.head_dim * self.dtype.itemsize * self.layer_num
-        return n, n
+        rows, es = self.size + self.page_size, self.dtype.itemsize
+        k = sum(rows * h * d * es for h, d in zip(self.head_nums, self.head_dims))
+        v = sum(rows * h * d * es for h, d in zip(self.head_nums, self.v_head_dims))
+        return k, v
 
     def get_key_buffer(self, layer_id: int):
         return self.k_buffer[layer_id]
@@ -199,8 +236,9 @@ class MHATokenToKVPool:
         # inside the scatter kernel; any other mismatch is converted here like the reference does
         if cache_k.dtype != self.dtype and self.dtype not in (torch.float8_e5m2, torch.float8_e4m3fn):
             cache_k, cache_v = cache_k.to(self.dtype), cache_v.to(self.dtype)
-        ops.store_kv_rows(self.k_buffer[layer_id], loc, cache_k.view(-1, self.head_num, self.head_dim))
-        ops.store_kv_rows(self.v_buffer[layer_id], loc, cache_v.view(-1, self.head_num, self.head_dim))
+        heads = self.head_nums[layer_id]
+        ops.store_kv_rows(self.k_buffer[layer_id], loc, cache_k.view(-1, heads, self.head_dims[layer_id]))
+        ops.store_kv_rows(self.v_buffer[layer_id], loc, cache_v.view(-1, heads, self.v_head_dims[layer_id]))
 
 
 class MLATokenToKVPool:

@@ -43,6 +43,7 @@ class ForwardBatch:
     extend_start_loc: Optional[torch.Tensor] = None    # int32 [B]
     extend_seq_lens_cpu: Optional[List[int]] = None
     extend_prefix_lens_cpu: Optional[List[int]] = None
+    extend_logit_rows: Optional[torch.Tensor] = None   # int64 rows of the flat token axis whose logits are wanted (None: last)
     # pools / backend
     req_to_token_pool: object = None
     token_to_kv_pool: object = None
@@ -77,6 +78,7 @@ class ForwardBatch:
                 ret.extend_prefix_lens, ret.extend_seq_lens, ret.extend_num_tokens)
             ret.extend_seq_lens_cpu = batch.extend_seq_lens
             ret.extend_prefix_lens_cpu = batch.extend_prefix_lens
+            ret.extend_logit_rows = getattr(batch, "extend_logit_rows", None)
         ret.req_to_token_pool = model_runner.req_to_token_pool
         ret.token_to_kv_pool = model_runner.token_to_kv_pool
         ret.attn_backend = model_runner.attn_backend

@@ -45,6 +45,9 @@ def build_model(model_config, dtype):
     if arch in ("DeepseekV2ForCausalLM", "DeepseekV3ForCausalLM"):
         from semi_pd_amd.models.deepseek_v2 import DeepseekV2ForCausalLM
         return DeepseekV2ForCausalLM(model_config, dtype)
+    if arch == "Kudirax":
+        from semi_pd_amd.models.kudirax import KudiraxForCausalLM
+        return KudiraxForCausalLM(model_config, dtype)
     raise ValueError(f"unsupported architecture {arch}")
 
 
@@ -224,9 +227,13 @@ class ModelRunner:
         self.model.eval()
         geo = self.model.kv_geometry
         self.kv_geometry = geo
-        self.num_attention_heads_local = geo["num_heads"]
-        self.num_kv_heads_local = geo["num_kv_heads"]
-        self.v_head_dim = geo["v_head_dim"]
+        # (a model whose layers differ gives lists, one entry per layer: the scalars the attention backend sizes its split
+        # buffers by are then the largest of each)
+        def largest(x):
+            return max(x) if isinstance(x, (list, tuple)) else x
+        self.num_attention_heads_local = largest(geo["num_heads"])
+        self.num_kv_heads_local = largest(geo["num_kv_heads"])
+        self.v_head_dim = largest(geo["v_head_dim"])
         self.sampler = Sampler()
 
         # ---- pools ---------------------------------------------------------------------------
@@ -277,6 +284,9 @@ class ModelRunner:
         geo = self.kv_geometry
         if geo["kind"] == "mla":
             cell = (geo["kv_lora_rank"] + geo["qk_rope_head_dim"]) * geo["num_layers"] * self.kv_cache_dtype.itemsize
+        elif isinstance(geo["num_kv_heads"], (list, tuple)):
+            cell = sum(h * (d + dv) for h, d, dv in zip(geo["num_kv_heads"], geo["head_dim"], geo["v_head_dim"])) \
+                * self.kv_cache_dtype.itemsize
         else:
             cell = (geo["num_kv_heads"] * (geo["head_dim"] + geo["v_head_dim"]) * geo["num_layers"]
                     * self.kv_cache_dtype.itemsize)
@@ -307,7 +317,7 @@ class ModelRunner:
         else:
             self.token_to_kv_pool = MHATokenToKVPool(self.max_total_num_tokens, 1, self.kv_cache_dtype,
                                                      geo["num_kv_heads"], geo["head_dim"], geo["num_layers"],
-                                                     dev, bypass_create_buffers=bypass)
+                                                     dev, bypass_create_buffers=bypass, v_head_dim=geo["v_head_dim"])
         self.token_to_kv_pool_allocator = TokenToKVPoolAllocator(self.max_total_num_tokens, self.kv_cache_dtype, dev,
                                                                  self.token_to_kv_pool)
 
@@ -360,6 +370,10 @@ class ModelRunner:
                 kv_handles.append([get_ipc_handle(pool.k_buffer[i]), get_ipc_handle(pool.v_buffer[i])])
             kv_info = {"kind": "mha", "shape": tuple(pool.k_buffer[0].shape), "dtype": pool.dtype,
                        "numel": pool.k_buffer[0].numel(), "layer_num": pool.layer_num}
+            if not pool.uniform:
+                # layers of their own geometry, values narrower or wider than keys: one shape per buffer
+                kv_info["shapes"] = [[tuple(pool.k_buffer[i].shape), tuple(pool.v_buffer[i].shape)]
+                                     for i in range(pool.layer_num)]
         else:
             for i in range(pool.layer_num):
                 kv_handles.append([get_ipc_handle(pool.kv_buffer[i])])
@@ -413,7 +427,15 @@ class ModelRunner:
         kvi = ipc_info.kvcache_info
         info = {"numel": kvi["numel"], "dtype": kvi["dtype"], "shape": kvi["shape"], "contiguous": True}
         pool = self.token_to_kv_pool
-        if kvi["kind"] == "mha":
+        if kvi["kind"] == "mha" and kvi.get("shapes"):
+            def one(handle, shape):
+                n = 1
+                for d in shape:
+                    n *= d
+                return self._import(handle, {"numel": n, "dtype": kvi["dtype"], "shape": tuple(shape), "contiguous": True})
+            pool.k_buffer = [one(h[0], sh[0]) for h, sh in zip(ipc_info.kv_cache_handles, kvi["shapes"])]
+            pool.v_buffer = [one(h[1], sh[1]) for h, sh in zip(ipc_info.kv_cache_handles, kvi["shapes"])]
+        elif kvi["kind"] == "mha":
             pool.k_buffer = [self._import(h[0], info) for h in ipc_info.kv_cache_handles]
             pool.v_buffer = [self._import(h[1], info) for h in ipc_info.kv_cache_handles]
         else:

@@ -25,18 +25,23 @@ from torch import nn
 def _config_classes():
     from semi_pd_amd.models.deepseek_v2 import DeepseekV2Config
     from semi_pd_amd.models.llama import LlamaConfig
+    from semi_pd_amd.models.kudirax import KudiraxConfig
     from semi_pd_amd.models.opt import OPTConfig
     return {"LlamaForCausalLM": LlamaConfig, "OPTForCausalLM": OPTConfig,
-            "DeepseekV2ForCausalLM": DeepseekV2Config, "DeepseekV3ForCausalLM": DeepseekV2Config}
+            "DeepseekV2ForCausalLM": DeepseekV2Config, "DeepseekV3ForCausalLM": DeepseekV2Config,
+            "Kudirax": KudiraxConfig}
 
 
 def config_from_hf_dict(d: dict):
-    archs = d.get("architectures") or []
+    # HF checkpoints list "architectures"; a config.json of this project's own designs names one "architecture"
+    archs = d.get("architectures") or ([d["architecture"]] if d.get("architecture") else [])
     classes = _config_classes()
     arch = next((a for a in archs if a in classes), None)
     if arch is None:
         raise ValueError(f"unsupported architectures {archs}; supported: {sorted(classes)}")
     cls = classes[arch]
+    if hasattr(cls, "from_dict"):
+        return cls.from_dict(d)      # nested per-layer configuration: the class reads its own keys
     if arch == "OPTForCausalLM" and d.get("word_embed_proj_dim", d.get("hidden_size")) != d.get("hidden_size"):
         raise ValueError("OPT checkpoints with word_embed_proj_dim != hidden_size are not supported")
     names = {f.name for f in dataclasses.fields(cls)}
@@ -98,12 +103,55 @@ class _Stacker:
 
 _QKV = {"q_proj": 0, "k_proj": 1, "v_proj": 2}
 _GATE_UP = {"gate_proj": 0, "up_proj": 1}
+_KUDIRAX_RE = re.compile(r"^l(\d+)\.(mix|mlp|norm1|norm2)(?:\.(.+))?$")
+_KUDIRAX_MERGED = {"q": 0, "k": 1, "v": 2, "g": 3}
+
+
+def _kudirax_items(config, weights):
+    """Kudirax checkpoint names (embed, l<i>.mix.q ..., l<i>.norm1[.b], l<i>.mlp.up[.b] ..., final.norm[.b], head) ->
+    product parameters; q | k | v | g stack into the mixer's merged projection."""
+    st = _Stacker()
+    top = {"embed": "embed.weight", "head": "head.weight", "final.norm": "final_norm.weight", "final.norm.b": "final_norm.bias"}
+    for name, t in weights:
+        if name in top:
+            yield top[name], t
+            continue
+        m = _KUDIRAX_RE.match(name)
+        if not m:
+            raise KeyError(f"checkpoint tensor {name} has no counterpart in a Kudirax model")
+        i, part, leaf = int(m.group(1)), m.group(2), m.group(3)
+        base = f"layers.{i}."
+        if part in ("norm1", "norm2"):
+            if part == "norm2" and not config.layers[i].ff:
+                continue                      # a layer without feed-forward has no second norm to apply
+            yield base + part + (".bias" if leaf == "b" else ".weight"), t
+        elif part == "mix":
+            if leaf in _KUDIRAX_MERGED:
+                yield from st.add(base + "mix.qkvg_proj.weight", _KUDIRAX_MERGED[leaf], 4, t)
+            elif leaf == "o":
+                yield base + "mix.o_proj.weight", t
+            elif leaf in ("sink", "vmix"):
+                yield base + "mix." + leaf, t
+            else:
+                raise KeyError(f"checkpoint tensor {name} has no counterpart in a Kudirax model")
+        else:
+            which, _, b = leaf.partition(".")
+            if which not in ("up", "down") or b not in ("", "b"):
+                raise KeyError(f"checkpoint tensor {name} has no counterpart in a Kudirax model")
+            yield base + f"mlp.{which}." + ("bias" if b else "weight"), t
+    if st.pending:
+        raise RuntimeError(f"checkpoint ended with incomplete stacked parameters: {list(st.pending)[:4]}")
+
+
 _EXPERT_RE = re.compile(r"^(.*\.mlp\.experts)\.(\d+)\.(gate_proj|up_proj|down_proj)\.(weight|weight_scale_inv)$")
 
 
 def product_items(config, weights: Iterable[Tuple[str, torch.Tensor]]) -> Iterator[Tuple[str, torch.Tensor]]:
     """HF tensor names -> (product parameter name, full unsharded tensor)."""
     arch = config.architectures[0]
+    if arch == "Kudirax":
+        yield from _kudirax_items(config, weights)
+        return
     st = _Stacker()
     tie = bool(getattr(config, "tie_word_embeddings", False))
     n_exp = int(getattr(config, "n_routed_experts", 0) or 0)

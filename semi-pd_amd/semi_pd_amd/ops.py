@@ -1282,3 +1282,123 @@ def moe_grouped_gemm_fp8(a_q: torch.Tensor, a_s: torch.Tensor, w_q: torch.Tensor
                                           N, K, sorted_token_ids.numel(), top_k_div, int(mul_routed_weight), block_m,
                                           int(block_shape[0]), int(block_shape[1]), dtype_code(c.dtype),
                                           current_stream(c.device)), "moe_grouped_gemm_fp8")
+
+
+# --------------------------------------------------------------------------- block-local attention with a sink term
+def unit_norm_and_store_kv(qkv: torch.Tensor, num_q_heads: int, num_kv_heads: int, qk_dim: int, v_dim: int, k_off: int,
+                           v_off: int, eps: float, k_buffer: torch.Tensor, v_buffer: torch.Tensor, loc: torch.Tensor,
+                           v_first: Optional[torch.Tensor] = None, mix: Optional[torch.Tensor] = None) -> None:
+    """Rows of `qkv` [T, >= v_off + G * v_dim] hold q | k | v at columns 0, k_off, v_off.  Per head q and k are divided by
+    their root mean square (eps inside the root, fp32): q in place, k into k_buffer[loc]; v -- blended as
+    (1 - mix) v + mix v_first where v_first [T, G * v_dim] is given -- into v_buffer[loc].  One launch
+    (csrc/local_attention.hip)."""
+    if qkv.dim() != 2 or qkv.stride(1) != 1:
+        raise RuntimeError("unit_norm_and_store_kv: qkv must be 2-D with contiguous rows")
+    T = qkv.shape[0]
+    if loc.dtype != torch.int64:
+        loc = loc.long()
+    if loc.shape[0] != T:
+        raise RuntimeError("unit_norm_and_store_kv: one pool slot per row")
+    for buf, size, name in ((k_buffer, qk_dim, "k_buffer"), (v_buffer, v_dim, "v_buffer")):
+        if buf.dtype != qkv.dtype or buf.dim() != 3 or buf.shape[1] != num_kv_heads or buf.shape[2] != size \
+                or not buf.is_contiguous():
+            raise RuntimeError(f"unit_norm_and_store_kv: {name} must be a contiguous [N, {num_kv_heads}, {size}] pool of "
+                               f"{qkv.dtype}, got {tuple(buf.shape)} {buf.dtype}")
+    if (v_first is None) != (mix is None):
+        raise RuntimeError("unit_norm_and_store_kv: v_first and mix come together")
+    if v_first is not None:
+        if v_first.dtype != qkv.dtype or v_first.shape != (T, num_kv_heads * v_dim) or v_first.stride(1) != 1:
+            raise RuntimeError("unit_norm_and_store_kv: v_first must be [T, kv heads * v_dim] of the activation type")
+        if mix.dtype != qkv.dtype or mix.numel() != 1:
+            raise RuntimeError("unit_norm_and_store_kv: mix is one element of the activation type")
+    if qkv.shape[1] < v_off + num_kv_heads * v_dim:
+        raise RuntimeError("unit_norm_and_store_kv: rows too short for the column offsets")
+    lib = _lib.load()
+    check(lib.semipd_unit_norm_kv_store(ptr(qkv), qkv.stride(0), T, num_q_heads, num_kv_heads, qk_dim, v_dim, k_off, v_off,
+                                        float(eps), ptr(v_first), v_first.stride(0) if v_first is not None else 0, ptr(mix),
+                                        ptr(k_buffer), ptr(v_buffer), ptr(loc), dtype_code(qkv.dtype),
+                                        current_stream(qkv.device)), "unit_norm_kv_store")
+
+
+def local_attention_mfma_supported(num_q_heads: int, num_kv_heads: int, qk_dim: int, v_dim: int, dtype: torch.dtype) -> bool:
+    return bool(_lib.load().semipd_local_attention_mfma_supported(num_q_heads, num_kv_heads, qk_dim, v_dim, dtype_code(dtype)))
+
+
+def local_attention_fwd(q: torch.Tensor, out: torch.Tensor, k_buffer: torch.Tensor, v_buffer: torch.Tensor,
+                        req_to_token: torch.Tensor, req_pool_indices: torch.Tensor, seq_lens: torch.Tensor,
+                        q_start: Optional[torch.Tensor], q_len: Optional[torch.Tensor], max_q_len: int, sm_scale: float,
+                        logit_cap: float = 0.0, chunk: int = 0, sink: Optional[torch.Tensor] = None,
+                        gate: Optional[torch.Tensor] = None, form: int = 0) -> None:
+    """Attention over the paged pools for prompt portions and decode steps alike (csrc/local_attention.hip).
+    q [T, H * D] and out / gate [T, H * E] may be column ranges of wider rows; k_buffer [N, G, D], v_buffer [N, G, E].
+    Request b owns rows q_start[b] .. + q_len[b], the last of them at position seq_lens[b] - 1; q_start None: one row per
+    request.  A query at position p sees the keys of its own block of `chunk` positions up to p (chunk 0: all up to p);
+    scores are capped by logit_cap * tanh(. / logit_cap); `sink` [H] fp32 adds exp(sink) to each head's denominator;
+    `gate`: out *= sigmoid(gate)."""
+    T = q.shape[0]
+    G, D = k_buffer.shape[1], k_buffer.shape[2]
+    E = v_buffer.shape[2]
+    if q.dim() != 2 or out.dim() != 2 or q.stride(1) != 1 or out.stride(1) != 1 or q.shape[1] % D or out.shape[1] % E:
+        raise RuntimeError("local_attention_fwd: q / out are [T, heads * size] with contiguous rows")
+    H = q.shape[1] // D
+    if out.shape != (T, H * E) or out.dtype != q.dtype or k_buffer.dtype != q.dtype or v_buffer.dtype != q.dtype:
+        raise RuntimeError("local_attention_fwd: shapes or types of q, out and the pools disagree")
+    if not (k_buffer.is_contiguous() and v_buffer.is_contiguous()) or v_buffer.shape[1] != G:
+        raise RuntimeError("local_attention_fwd: pools must be contiguous [N, G, size]")
+    if gate is not None and (gate.shape != out.shape or gate.dtype != q.dtype or gate.stride(1) != 1):
+        raise RuntimeError("local_attention_fwd: gate must look like out")
+    if sink is not None and (sink.dtype != torch.float32 or sink.numel() != H or not sink.is_contiguous()):
+        raise RuntimeError("local_attention_fwd: sink is fp32 [H]")
+    if req_to_token.dtype != torch.int32 or req_pool_indices.dtype != torch.int64 or seq_lens.dtype != torch.int64:
+        raise RuntimeError("local_attention_fwd: req_to_token int32, req_pool_indices / seq_lens int64")
+    B = req_pool_indices.shape[0]
+    if (q_start is None) != (q_len is None):
+        raise RuntimeError("local_attention_fwd: q_start and q_len come together")
+    if q_start is not None and (q_start.dtype != torch.int32 or q_len.dtype != torch.int32
+                                or q_start.shape[0] != B or q_len.shape[0] != B):
+        raise RuntimeError("local_attention_fwd: q_start / q_len are int32 [B]")
+    if q_start is None and T != B:
+        raise RuntimeError("local_attention_fwd: one query row per request when q_start is None")
+    lib = _lib.load()
+    check(lib.semipd_local_attention(ptr(q), q.stride(0), ptr(gate), gate.stride(0) if gate is not None else 0, ptr(out),
+                                     out.stride(0), ptr(k_buffer), ptr(v_buffer), ptr(req_to_token), req_to_token.stride(0),
+                                     ptr(req_pool_indices), ptr(seq_lens), ptr(q_start), ptr(q_len), B, T, int(max_q_len), H, G,
+                                     D, E, ptr(sink), float(sm_scale), float(logit_cap), int(chunk), int(form),
+                                     dtype_code(q.dtype), current_stream(q.device)), "local_attention")
+
+
+# --------------------------------------------------------------------------- LayerNorm of post-norm blocks, squared ReLU
+def layernorm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float,
+              residual: Optional[torch.Tensor] = None, in_bias: Optional[torch.Tensor] = None,
+              out_dtype: Optional[torch.dtype] = None, want_out: bool = True) -> Optional[torch.Tensor]:
+    """LayerNorm(x + in_bias) * weight + bias per row in fp32 (csrc/layernorm.hip); x rows fp32 or of the parameters' type.
+    `residual` (fp32 [rows, width], updated in place): the result is added to it and the sum is returned in the
+    parameters' type (None with want_out=False)."""
+    dt = weight.dtype
+    if x.dim() != 2 or x.stride(1) != 1 or x.dtype not in (dt, torch.float32):
+        raise RuntimeError("layernorm: x must be 2-D with contiguous rows, fp32 or of the weight's type")
+    rows, width = x.shape
+    if weight.shape != (width,) or bias.shape != (width,) or bias.dtype != dt or (in_bias is not None and (
+            in_bias.shape != (width,) or in_bias.dtype != dt)):
+        raise RuntimeError("layernorm: weight / bias / in_bias are [width] of one type")
+    if residual is not None and (residual.dtype != torch.float32 or residual.shape != x.shape or residual.stride(1) != 1):
+        raise RuntimeError("layernorm: residual is fp32 and shaped like x")
+    if out_dtype is not None and out_dtype != dt:
+        raise RuntimeError("layernorm: the output has the parameters' type")
+    out = torch.empty((rows, width), dtype=dt, device=x.device) if (want_out or residual is None) else None
+    lib = _lib.load()
+    check(lib.semipd_layernorm(ptr(x), x.stride(0), 1 if (x.dtype == torch.float32 and dt != torch.float32) else 0, ptr(in_bias),
+                               ptr(weight), ptr(bias), float(eps), ptr(residual), residual.stride(0) if residual is not None else 0,
+                               ptr(out), out.stride(0) if out is not None else 0, rows, width, dtype_code(dt),
+                               current_stream(x.device)), "layernorm")
+    return out
+
+
+def bias_relu_square_(u: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """u <- max(u + bias, 0)^2 in place (csrc/layernorm.hip)."""
+    if u.dim() != 2 or u.stride(1) != 1 or (bias is not None and (bias.shape != (u.shape[1],) or bias.dtype != u.dtype)):
+        raise RuntimeError("bias_relu_square_: u is 2-D with contiguous rows, bias [width] of the same type")
+    lib = _lib.load()
+    check(lib.semipd_bias_relu_square(ptr(u), u.stride(0), ptr(bias), u.shape[0], u.shape[1], dtype_code(u.dtype),
+                                      current_stream(u.device)), "bias_relu_square")
+    return u

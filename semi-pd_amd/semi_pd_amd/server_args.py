@@ -151,7 +151,8 @@ class ServerArgs:
 
     @property
     def torch_dtype(self) -> torch.dtype:
-        return {"bfloat16": torch.bfloat16, "float16": torch.float16, "half": torch.float16}[self.dtype]
+        return {"bfloat16": torch.bfloat16, "float16": torch.float16, "half": torch.float16,
+                "float32": torch.float32}[self.dtype]
 
 
 @dataclasses.dataclass
@@ -188,7 +189,7 @@ def add_cli_args(parser):
     p.add_argument("--port", type=int, default=30000)
     p.add_argument("--skip-tokenizer-init", action="store_true")
     p.add_argument("--load-format", type=str, default="auto", choices=["auto", "safetensors", "dummy"])
-    p.add_argument("--dtype", type=str, default="auto", choices=["auto", "half", "float16", "bfloat16"])
+    p.add_argument("--dtype", type=str, default="auto", choices=["auto", "half", "float16", "bfloat16", "float32"])
     p.add_argument("--kv-cache-dtype", type=str, default="auto", choices=["auto", "fp8_e5m2", "fp8_e4m3"])
     p.add_argument("--context-length", type=int, default=None)
     p.add_argument("--served-model-name", type=str, default=None)
