@@ -171,9 +171,315 @@ __global__ void __launch_bounds__(256) local_attention_rows_kernel(LocalAttnArgs
   }
 }
 
+// ------------------------------------------------------------------------------------------------ matrix-core forms
+// v_mfma_f32_16x16x32 (lane l: r = l & 15, g = l >> 4): a = A[row r][k 8g .. 8g+7], b = B[k 8g .. 8g+7][col r],
+// d[i] = D[row 4g + i][col r].  One step covers 32 keys: S^T = K Q^T is taken in two 16-row groups whose row rho stands
+// for key 8 (rho / 4) + rho % 4 (group A) and that key + 4 (group B), so that lane (r, g) ends up with the scores of keys
+// 8g .. 8g+7 of query r -- which is the b operand of O^T += V^T P^T as it stands.  V^T comes from an LDS tile [E][32].
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+constexpr int kVtLd = 40;                     // elements per V^T row in LDS: 32 keys + 8 of padding (80 bytes)
+
+template <typename T> __device__ __forceinline__ f32x4 mma16(const Frag16& a, const Frag16& b, f32x4 c);
+template <> __device__ __forceinline__ f32x4 mma16<bf16_t>(const Frag16& a, const Frag16& b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, b.b, c, 0, 0, 0);
+}
+template <> __device__ __forceinline__ f32x4 mma16<f16_t>(const Frag16& a, const Frag16& b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(a.f, b.f, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ float fast_capped(float s, float scale, float cap) {
+  s *= scale;
+  if (cap > 0.f) {
+    const float e = __expf(2.0f * s / cap);   // tanh(x) = 1 - 2 / (exp(2x) + 1); exp overflow gives 1, underflow -1
+    s = cap * (1.0f - 2.0f / (e + 1.0f));
+  }
+  return s;
+}
+
+// 32 rows of V (keys j0 .. j0+31 of the request, rows past `hi` as zeros) -> vt[e][key], by NT threads
+template <typename T, int NT>
+__device__ __forceinline__ void stage_vt(T* vt, const T* vp, const int32_t* row, int64_t j0, int64_t hi, int G, int gk, int E,
+                                         int tid) {
+  const int per_key = E >> 3;
+  for (int c = tid; c < 32 * per_key; c += NT) {
+    const int key = c / per_key, ec = c - key * per_key;
+    const int64_t j = j0 + key;
+    Vec16<T> v;
+    if (j <= hi) {
+      v = load16(vp + ((int64_t)row[j] * G + gk) * E + ec * 8);
+    } else {
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v.e[u].v = 0;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) vt[(ec * 8 + u) * kVtLd + key] = v.e[u];
+  }
+}
+
+template <int NE> struct SoftState {
+  float m, l;
+  f32x4 acc[NE];
+};
+
+// One step of 32 keys for the 16 columns of this wave.  sa / sb: the raw dot products of groups A and B (4 each) are
+// turned into probabilities against the running maximum, the accumulators are rescaled and V^T P^T is added.
+// ok(i): whether key 8g + i of the step is visible to this lane's column.
+template <typename T, int NE, typename Ok>
+__device__ __forceinline__ void soft_step(SoftState<NE>& st, f32x4 sa, f32x4 sb, float scale, float cap, Ok ok, const T* vt, int ne,
+                                          int r, int g) {
+  float s[8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    s[i] = ok(i) ? fast_capped(sa[i], scale, cap) : -INFINITY;
+    s[4 + i] = ok(4 + i) ? fast_capped(sb[i], scale, cap) : -INFINITY;
+  }
+  float mt = s[0];
+#pragma unroll
+  for (int i = 1; i < 8; ++i) mt = fmaxf(mt, s[i]);
+  mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
+  mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+  const float m_new = fmaxf(st.m, mt);
+  const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+  const float alpha = __expf(st.m - m_safe);         // st.m = -inf: 0, and nothing has been accumulated yet
+  float p[8], sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    p[i] = __expf(s[i] - m_safe);
+    sum += p[i];
+  }
+  st.l = st.l * alpha + sum;
+  st.m = m_new;
+  Frag16 pb;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) pb.w[i] = pack2<T>(p[2 * i], p[2 * i + 1]);
+#pragma unroll
+  for (int eb = 0; eb < NE; ++eb) {
+    if (eb < ne) {
+      Frag16 va;
+      va.u = *reinterpret_cast<const uint4*>(vt + (eb * 16 + r) * kVtLd + 8 * g);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) st.acc[eb][i] *= alpha;
+      st.acc[eb] = mma16<T>(va, pb, st.acc[eb]);
+    }
+  }
+}
+
+// the two groups of K rows of a step against the wave's Q fragments
+template <typename T, int ND>
+__device__ __forceinline__ void score_step(const Frag16 (&qf)[ND], int nd, const T* ka, const T* kb, int g, f32x4& sa, f32x4& sb) {
+  sa = f32x4{0.f, 0.f, 0.f, 0.f};
+  sb = f32x4{0.f, 0.f, 0.f, 0.f};
+  Frag16 fa[ND], fb[ND];
+#pragma unroll
+  for (int kk = 0; kk < ND; ++kk)
+    if (kk < nd) {
+      fa[kk].u = *reinterpret_cast<const uint4*>(ka + 32 * kk + 8 * g);
+      fb[kk].u = *reinterpret_cast<const uint4*>(kb + 32 * kk + 8 * g);
+    }
+#pragma unroll
+  for (int kk = 0; kk < ND; ++kk)
+    if (kk < nd) {
+      sa = mma16<T>(fa[kk], qf[kk], sa);
+      sb = mma16<T>(fb[kk], qf[kk], sb);
+    }
+}
+
+// Prompt portions: 64 query rows of one request and one head per workgroup, 16 per wave.
+template <typename T, int ND, int NE>
+__global__ void __launch_bounds__(256) local_attention_mfma_kernel(LocalAttnArgs a) {
+  __shared__ __attribute__((aligned(16))) T vt[NE * 16 * kVtLd];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
+  const int h = blockIdx.y;
+  // which request and which 64-row tile of it
+  int b = -1;
+  int64_t q0 = 0;
+  {
+    int64_t left = blockIdx.x;
+    for (int rq = 0; rq < (int)a.batch; ++rq) {
+      const int64_t tiles = ((int64_t)a.q_len[rq] + 63) >> 6;
+      if (left < tiles) {
+        b = rq;
+        q0 = left << 6;
+        break;
+      }
+      left -= tiles;
+    }
+  }
+  if (b < 0) return;
+  const int D = a.D, E = a.E, G = a.G, nd = D >> 5, ne = E >> 4;
+  const int gk = h / (a.H / G);
+  const int64_t qn = a.q_len[b], base_pos = a.seq_lens[b] - qn, t0 = a.q_start[b];
+  const int chunk = a.chunk;
+  auto lo_of = [&](int64_t p) -> int64_t { return chunk > 0 ? (p / chunk) * chunk : 0; };
+  const int64_t blk_last = (q0 + 63 < qn - 1 ? q0 + 63 : qn - 1);
+  const int64_t blk_lo = lo_of(base_pos + q0), blk_hi = base_pos + blk_last;
+  // this wave's 16 rows
+  const int64_t wq0 = q0 + 16 * wave;
+  const bool wave_on = wq0 < qn;
+  const int64_t wq_last = wq0 + 15 < qn - 1 ? wq0 + 15 : qn - 1;
+  const int64_t w_lo = lo_of(base_pos + wq0), w_hi = base_pos + wq_last;
+  const bool q_ok = wq0 + r < qn;
+  const int64_t my_q = q_ok ? wq0 + r : (wave_on ? wq_last : 0);
+  const int64_t my_pos = base_pos + my_q, my_lo = lo_of(my_pos);
+  Frag16 qf[ND];
+  {
+    const T* q = (const T*)a.q + (t0 + my_q) * a.q_ld + (int64_t)h * D;
+#pragma unroll
+    for (int kk = 0; kk < ND; ++kk)
+      if (kk < nd) qf[kk].u = *reinterpret_cast<const uint4*>(q + 32 * kk + 8 * g);
+  }
+  SoftState<NE> st;
+  st.m = -INFINITY;
+  st.l = 0.f;
+#pragma unroll
+  for (int eb = 0; eb < NE; ++eb) st.acc[eb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int32_t* row = a.req_to_token + a.req_pool_indices[b] * a.r2t_stride;
+  const T* kp = (const T*)a.k_pool + (int64_t)gk * D;
+  const T* vp = (const T*)a.v_pool;
+  const int64_t kstride = (int64_t)G * D;
+  const int ka_off = 8 * (r >> 2) + (r & 3);
+  for (int64_t j0 = blk_lo; j0 <= blk_hi; j0 += 32) {
+    __syncthreads();                                   // everyone is done with the previous V^T tile
+    stage_vt<T, 256>(vt, vp, row, j0, blk_hi, G, gk, E, tid);
+    __syncthreads();
+    if (!wave_on || j0 + 31 < w_lo || j0 > w_hi) continue;
+    const int64_t ja = j0 + ka_off, jb = ja + 4;
+    const T* ka = kp + (int64_t)(ja <= blk_hi ? row[ja] : 0) * kstride;
+    const T* kb = kp + (int64_t)(jb <= blk_hi ? row[jb] : 0) * kstride;
+    f32x4 sa, sb;
+    score_step<T, ND>(qf, nd, ka, kb, g, sa, sb);
+    const int64_t jl = j0 + 8 * g;
+    soft_step<T, NE>(st, sa, sb, a.scale, a.cap,
+                     [&](int i) { const int64_t j = jl + i; return q_ok && j >= my_lo && j <= my_pos; }, vt, ne, r, g);
+  }
+  if (!q_ok) {
+    // (rows past the request's end took part in the shuffles above only)
+  }
+  float l = st.l;
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (!q_ok) return;
+  if (a.sink != nullptr) l += __expf(a.sink[h] - st.m);
+  const float inv = 1.0f / l;
+  T* o = (T*)a.out + (t0 + my_q) * a.out_ld + (int64_t)h * E;
+  const T* gt = a.gate ? (const T*)a.gate + (t0 + my_q) * a.gate_ld + (int64_t)h * E : nullptr;
+#pragma unroll
+  for (int eb = 0; eb < NE; ++eb)
+    if (eb < ne) {
+      const int e0 = eb * 16 + 4 * g;
+      float y[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        y[i] = st.acc[eb][i] * inv;
+        if (gt) y[i] *= 1.0f / (1.0f + __expf(-Elem<T>::to_f(gt[e0 + i])));
+      }
+      uint2 w;
+      w.x = pack2<T>(y[0], y[1]);
+      w.y = pack2<T>(y[2], y[3]);
+      *reinterpret_cast<uint2*>(o + e0) = w;
+    }
+}
+
+// Decode steps: one workgroup per (request, kv head, group of 16 q heads); the q heads are the 16 columns, the four waves
+// take the 32-key steps in turn and meet in LDS.
+template <typename T, int ND, int NE>
+__global__ void __launch_bounds__(256) local_attention_decode_kernel(LocalAttnArgs a) {
+  __shared__ __attribute__((aligned(16))) T vt[4][NE * 16 * kVtLd];
+  __shared__ float part_ml[4][2][16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
+  const int b = blockIdx.x, gk = blockIdx.y;
+  const int D = a.D, E = a.E, G = a.G, nd = D >> 5, ne = E >> 4;
+  const int rep = a.H / G;
+  const int col0 = blockIdx.z * 16;
+  const bool col_ok = col0 + r < rep;
+  const int h = gk * rep + (col_ok ? col0 + r : col0);
+  const int64_t t = a.q_start ? (int64_t)a.q_start[b] + a.q_len[b] - 1 : b;     // the request's newest row
+  const int64_t pos = a.seq_lens[b] - 1;
+  if (pos < 0) return;
+  const int64_t lo = a.chunk > 0 ? (pos / a.chunk) * a.chunk : 0;
+  Frag16 qf[ND];
+  {
+    const T* q = (const T*)a.q + t * a.q_ld + (int64_t)h * D;
+#pragma unroll
+    for (int kk = 0; kk < ND; ++kk)
+      if (kk < nd) qf[kk].u = *reinterpret_cast<const uint4*>(q + 32 * kk + 8 * g);
+  }
+  SoftState<NE> st;
+  st.m = -INFINITY;
+  st.l = 0.f;
+#pragma unroll
+  for (int eb = 0; eb < NE; ++eb) st.acc[eb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int32_t* row = a.req_to_token + a.req_pool_indices[b] * a.r2t_stride;
+  const T* kp = (const T*)a.k_pool + (int64_t)gk * D;
+  const T* vp = (const T*)a.v_pool;
+  const int64_t kstride = (int64_t)G * D;
+  const int ka_off = 8 * (r >> 2) + (r & 3);
+  for (int64_t j0 = lo + 32 * wave; j0 <= pos; j0 += 128) {
+    // the wave's own V^T tile: its LDS accesses are executed in order, the barrier keeps the compiler from mixing them
+    __builtin_amdgcn_wave_barrier();
+    stage_vt<T, 64>(vt[wave], vp, row, j0, pos, G, gk, E, lane);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int64_t ja = j0 + ka_off, jb = ja + 4;
+    const T* ka = kp + (int64_t)(ja <= pos ? row[ja] : 0) * kstride;
+    const T* kb = kp + (int64_t)(jb <= pos ? row[jb] : 0) * kstride;
+    f32x4 sa, sb;
+    score_step<T, ND>(qf, nd, ka, kb, g, sa, sb);
+    const int64_t jl = j0 + 8 * g;
+    soft_step<T, NE>(st, sa, sb, a.scale, a.cap, [&](int i) { return jl + i <= pos; }, vt[wave], ne, r, g);
+  }
+  float l = st.l;
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (g == 0) {
+    part_ml[wave][0][r] = st.m;
+    part_ml[wave][1][r] = l;
+  }
+  // a wave's partial sums go where its V^T tile was ([e][17] floats fit in [e][40] halves); only the wave itself read it
+  __builtin_amdgcn_wave_barrier();
+  float* mine = reinterpret_cast<float*>(vt[wave]);
+#pragma unroll
+  for (int eb = 0; eb < NE; ++eb)
+    if (eb < ne)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) mine[(eb * 16 + 4 * g + i) * 17 + r] = st.acc[eb][i];
+  __syncthreads();
+  // merge: thread (column c, slice) walks the value elements slice, slice + 16, ...
+  const int c = tid & 15, slice = tid >> 4;
+  if (col0 + c >= rep) return;
+  float m = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) m = fmaxf(m, part_ml[w][0][c]);
+  float f[4], lt = 0.f;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const float mw = part_ml[w][0][c];
+    f[w] = mw == -INFINITY ? 0.f : __expf(mw - m);
+    lt += f[w] * part_ml[w][1][c];
+  }
+  const int hh = gk * rep + col0 + c;
+  if (a.sink != nullptr) lt += __expf(a.sink[hh] - m);
+  const float inv = 1.0f / lt;
+  T* o = (T*)a.out + t * a.out_ld + (int64_t)hh * E;
+  const T* gt = a.gate ? (const T*)a.gate + t * a.gate_ld + (int64_t)hh * E : nullptr;
+  for (int e = slice; e < E; e += 16) {
+    float y = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) y += f[w] * reinterpret_cast<const float*>(vt[w])[e * 17 + c];
+    y *= inv;
+    if (gt) y *= 1.0f / (1.0f + __expf(-Elem<T>::to_f(gt[e])));
+    o[e] = Elem<T>::from_f(y);
+  }
+}
+
 }  // namespace semipd
 
 using namespace semipd;
+
+static inline bool local_mfma_shape_ok(int qk_dim, int v_dim) {
+  return qk_dim % 32 == 0 && qk_dim <= 256 && v_dim % 16 == 0 && v_dim <= 256;
+}
 
 extern "C" int semipd_unit_norm_kv_store(void* qkv, int64_t ld, int64_t num_tokens, int num_q_heads, int num_kv_heads,
                                          int qk_dim, int v_dim, int64_t k_off, int64_t v_off, float eps, const void* v_first,
@@ -218,8 +524,33 @@ extern "C" int semipd_local_attention(const void* q, int64_t q_ld, const void* g
   LocalAttnArgs a{q, q_ld, gate, gate_ld, out, out_ld, k_pool, v_pool, req_to_token, req_to_token_stride, req_pool_indices,
                   seq_lens, q_start, q_len, batch, num_tokens, num_q_heads, num_kv_heads, qk_dim, v_dim, sink, scale, logit_cap,
                   chunk};
-  (void)max_q_len;
-  (void)form;
+  const bool half = dtype == SEMIPD_BF16 || dtype == SEMIPD_F16;
+  const bool mfma_ok = half && local_mfma_shape_ok(qk_dim, v_dim) && aligned16(q) && q_ld % 8 == 0 && aligned16(k_pool) &&
+                       aligned16(v_pool) && aligned16(out) && out_ld % 4 == 0;
+  SEMIPD_CHECK_ARG(form != 2 || mfma_ok, SEMIPD_ESHAPE, "local_attention: the matrix-core forms do not take this shape or type");
+  if (form != 1 && mfma_ok) {
+    const bool small = qk_dim <= 128 && v_dim <= 128;
+    if (q_start == nullptr || max_q_len <= 1) {
+      const dim3 grid((unsigned)batch, (unsigned)num_kv_heads, (unsigned)((num_q_heads / num_kv_heads + 15) / 16));
+      if (dtype == SEMIPD_BF16) {
+        if (small) hipLaunchKernelGGL((local_attention_decode_kernel<bf16_t, 4, 8>), grid, dim3(256), 0, as_stream(stream), a);
+        else hipLaunchKernelGGL((local_attention_decode_kernel<bf16_t, 8, 16>), grid, dim3(256), 0, as_stream(stream), a);
+      } else {
+        if (small) hipLaunchKernelGGL((local_attention_decode_kernel<f16_t, 4, 8>), grid, dim3(256), 0, as_stream(stream), a);
+        else hipLaunchKernelGGL((local_attention_decode_kernel<f16_t, 8, 16>), grid, dim3(256), 0, as_stream(stream), a);
+      }
+      return launch_status("local_attention_decode");
+    }
+    const dim3 grid((unsigned)((num_tokens + 63) / 64 + batch), (unsigned)num_q_heads);
+    if (dtype == SEMIPD_BF16) {
+      if (small) hipLaunchKernelGGL((local_attention_mfma_kernel<bf16_t, 4, 8>), grid, dim3(256), 0, as_stream(stream), a);
+      else hipLaunchKernelGGL((local_attention_mfma_kernel<bf16_t, 8, 16>), grid, dim3(256), 0, as_stream(stream), a);
+    } else {
+      if (small) hipLaunchKernelGGL((local_attention_mfma_kernel<f16_t, 4, 8>), grid, dim3(256), 0, as_stream(stream), a);
+      else hipLaunchKernelGGL((local_attention_mfma_kernel<f16_t, 8, 16>), grid, dim3(256), 0, as_stream(stream), a);
+    }
+    return launch_status("local_attention_mfma");
+  }
   const dim3 grid((unsigned)((num_tokens + 3) / 4), (unsigned)num_q_heads);
   SEMIPD_DISPATCH_DTYPE(dtype, T,
                         hipLaunchKernelGGL((local_attention_rows_kernel<T>), grid, dim3(256), 0, as_stream(stream), a));
@@ -227,6 +558,6 @@ extern "C" int semipd_local_attention(const void* q, int64_t q_ld, const void* g
 }
 
 extern "C" int semipd_local_attention_mfma_supported(int num_q_heads, int num_kv_heads, int qk_dim, int v_dim, int dtype) {
-  (void)num_q_heads; (void)num_kv_heads; (void)qk_dim; (void)v_dim; (void)dtype;
-  return 0;
+  return (dtype == SEMIPD_BF16 || dtype == SEMIPD_F16) && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0 &&
+         local_mfma_shape_ok(qk_dim, v_dim);
 }
