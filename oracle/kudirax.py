@@ -55,6 +55,19 @@ def sink_softmax(s: torch.Tensor, mask: torch.Tensor, sink: Optional[torch.Tenso
     return p[..., :-1]
 
 
+def local_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, cap: float, chunk: Optional[int],
+                    sink: Optional[torch.Tensor]) -> torch.Tensor:
+    """One whole sequence: q [T, H, D], k [T, G, D], v [T, G, E] -> [T, H, E].  Query head h reads key/value head
+    h // (H / G); capped scores; block-local causal mask; sink in the denominator."""
+    T, H = q.shape[0], q.shape[1]
+    rep = H // k.shape[1]
+    kk = k.float().repeat_interleave(rep, 1)
+    vv = v.float().repeat_interleave(rep, 1)
+    s = soft_cap(torch.einsum("ihd,jhd->hij", q.float(), kk) * scale, cap)
+    p = sink_softmax(s, visible(T, chunk), sink)
+    return torch.einsum("hij,jhe->ihe", p, vv)
+
+
 def attention_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], pre: str, m: dict, eps: float,
                     v_first: Optional[torch.Tensor]):
     """One sequence h [T, width] through the attention mixer whose tensors start with `pre`.
@@ -69,14 +82,8 @@ def attention_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], pre: str, m: di
     if v_first is not None:
         lam = w[pre + "vmix"].float()
         v = (1.0 - lam) * v + lam * v_first
-    rep = H // G
-    kk = k.repeat_interleave(rep, 1)
-    vv = v.repeat_interleave(rep, 1)
-    s = torch.einsum("ihd,jhd->hij", q, kk) * m["scale"]
-    s = soft_cap(s, m.get("softcap") or 0.0)
-    chunk = (m.get("mask") or {}).get("size")
-    p = sink_softmax(s, visible(T, chunk), w.get(pre + "sink"))
-    o = torch.einsum("hij,jhe->ihe", p, vv).reshape(T, H * E)
+    o = local_attention(q, k, v, m["scale"], m.get("softcap") or 0.0, (m.get("mask") or {}).get("size"),
+                        w.get(pre + "sink")).reshape(T, H * E)
     o = o * torch.sigmoid(h @ w[pre + "g"].float().T)
     return o @ w[pre + "o"].float().T, v
 
