@@ -492,7 +492,20 @@ def main():
                     "otherwise; '' = none")
     ap.add_argument("--sweep-output-len", type=int, default=SWEEP_OUTPUT_LEN, help="default: --output-len")
     ap.add_argument("--sweep-num-requests", type=int, default=None, help="requests per sweep point (default: --num-requests)")
+    ap.add_argument("--arch-compare", action="store_true",
+                    help="instead of the serving line: Kudirax next to Llama at equal layer sizes, models and kernels "
+                         "(tools/arch_compare.py); one JSON object of its own")
+    ap.add_argument("--arch-sizes", default="", help="--arch-compare: comma-separated size names (default: all)")
+    ap.add_argument("--arch-chunk", type=int, default=1024, help="--arch-compare: positions per attention block (0: none)")
     args = ap.parse_args()
+
+    if args.arch_compare:
+        import importlib.util
+        spec = importlib.util.spec_from_file_location("arch_compare", os.path.join(ROOT, "tools", "arch_compare.py"))
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        mod.main(args)
+        return
 
     if args.rate_sweep is None:
         default_workload = (args.gpus == 1 and args.model == "llama3-8b" and args.mode == "semi-pd"

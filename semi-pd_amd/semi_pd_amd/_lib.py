@@ -160,6 +160,54 @@ _RESTYPES = {"semipd_last_error": C.c_char_p, "semipd_lm_head_argmax_workspace":
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 
 
+# ---- building a part of the library ------------------------------------------------------------------------------------
+# The whole library is ~3 CPU-minutes of hipcc.  A process that serves ONE model in a checkout where nothing is built yet
+# (bin/trace_run) compiles the sources that model's path calls into and links them as a library of its own name; the
+# whole library, once built (`make -C semi-pd_amd/csrc`, __graft_entry__.build()), always takes precedence.
+CORE_SOURCES = ("elementwise.hip", "skinny_gemm.hip", "stream_linear.hip", "gemm8p.hip", "dense_gemm.hip", "moe.hip",
+                "moe_tiled_gemm.hip", "sampling.hip", "ipc.hip")          # pools, GEMMs, logits, sampler, streams
+MODEL_SOURCES = {
+    "Kudirax": ("local_attention.hip", "layernorm.hip"),
+}
+
+
+def ensure_library_for(architecture: str, log=None) -> str:
+    """Path of a library that holds every kernel `architecture` needs: the whole library if it is built, else a partial one
+    (built now if missing) for the architectures listed in MODEL_SOURCES, else the whole library, built now."""
+    import hashlib
+    import subprocess
+    csrc = os.path.join(os.path.dirname(_PKG_DIR), "csrc")
+    if os.environ.get("SEMIPD_HIP_LIB") or os.path.exists(LIB_PATH):
+        return LIB_PATH
+    jobs = str(max(1, min(16, len(os.sched_getaffinity(0)))))
+    extra = MODEL_SOURCES.get(architecture)
+    if extra is None:
+        cmd, path = ["make", "-C", csrc, "-j", jobs], LIB_PATH
+    else:
+        srcs = sorted(set(CORE_SOURCES + tuple(extra)))
+        tag = hashlib.sha256(" ".join(srcs).encode()).hexdigest()[:10]
+        path = os.path.join(os.path.dirname(LIB_PATH), f"libsemipd_hip.part-{tag}.so")
+        cmd = ["make", "-C", csrc, "-j", jobs, "SRCS=" + " ".join(srcs), "LIB=" + os.path.relpath(path, csrc)]
+    if not os.path.exists(path):
+        if log:
+            log(f"building {os.path.basename(path)} ({' '.join(cmd[4:]) or 'every source'})")
+        subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL)
+    return path
+
+
+def use_library(path: str) -> None:
+    """Load `path` instead of the default library (before the first load()).  A partial library binds the entry points it
+    has; calling one it lacks raises AttributeError naming the symbol."""
+    global LIB_PATH, _partial
+    if _lib is not None and path != LIB_PATH:
+        raise RuntimeError("the native library is already loaded")
+    _partial = ".part-" in os.path.basename(path)
+    LIB_PATH = path
+
+
+_partial = False
+
+
 def load() -> C.CDLL:
     """Load (once) and return the shared library; fail loudly if it is not built."""
     global _lib
@@ -176,6 +224,8 @@ def load() -> C.CDLL:
             )
         lib = C.CDLL(LIB_PATH)
         for name, argtypes in _SIGNATURES.items():
+            if _partial and not hasattr(lib, name):
+                continue             # not in this partial library: a call raises AttributeError (undefined symbol)
             fn = getattr(lib, name)  # AttributeError = header / library mismatch
             fn.argtypes = argtypes
             fn.restype = _RESTYPES.get(name, C.c_int)

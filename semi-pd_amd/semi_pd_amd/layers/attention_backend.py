@@ -247,11 +247,12 @@ class HipAttnBackend(AttentionBackend):
 
 
     # ---- block-local attention with a sink term: prompt portions and decode steps over the pools -------------------
-    def forward_local(self, q, layer, forward_batch: ForwardBatch, gate=None):
+    def forward_local(self, q, layer, forward_batch: ForwardBatch, gate=None, sink=None):
         """Attention for layers whose keys and values are in the pool already (the model stored them with the step that
         prepares q): q [T, heads * head_dim] (may be a column range), keys found through req_to_token, so an extend batch
         -- whole prompts, portions with a cached prefix, single tokens of running requests side by side -- and a decode
-        batch are the same call.  Mask, cap and sink come from the layer descriptor; `gate` multiplies sigmoid(gate) in."""
+        batch are the same call.  Mask and cap come from the layer descriptor; `sink` (fp32 [heads], the module's parameter) adds
+        exp(sink) to each head's softmax denominator; `gate` multiplies sigmoid(gate) in."""
         T = q.shape[0]
         o = torch.empty((T, layer.tp_q_head_num * layer.v_head_dim), dtype=q.dtype, device=q.device)
         pool = forward_batch.token_to_kv_pool
@@ -265,7 +266,7 @@ class HipAttnBackend(AttentionBackend):
         t0 = kt.start() if kt else None
         ops.local_attention_fwd(q, o, pool.get_key_buffer(layer.layer_id), pool.get_value_buffer(layer.layer_id),
                                 self.req_to_token, forward_batch.req_pool_indices, forward_batch.seq_lens, q_start, q_len, max_q,
-                                layer.scaling, layer.logit_cap, layer.chunk_size, layer.sink, gate,
+                                layer.scaling, layer.logit_cap, layer.chunk_size, sink, gate,
                                 form=int(os.environ.get("SEMIPD_LOCAL_ATTN_FORM", "0")))
         if kt:
             kt.stop("decode_attention" if forward_batch.forward_mode.is_decode() else "extend_attention", t0, 0.0, 0.0)
@@ -336,7 +337,7 @@ class RadixAttention:
     layer id; forward() reshapes nothing and dispatches to the batch's backend."""
 
     def __init__(self, num_heads: int, head_dim: int, scaling: float, num_kv_heads: int, layer_id: int,
-                 logit_cap: float = 0.0, v_head_dim: int = -1, chunk_size: int = 0, sink: Optional[torch.Tensor] = None):
+                 logit_cap: float = 0.0, v_head_dim: int = -1, chunk_size: int = 0):
         self.tp_q_head_num = num_heads
         self.tp_k_head_num = num_kv_heads
         self.tp_v_head_num = num_kv_heads
@@ -347,10 +348,8 @@ class RadixAttention:
         self.layer_id = layer_id
         self.logit_cap = logit_cap
         # block-local attention (HipAttnBackend.forward_local): a query sees the keys of its own block of chunk_size positions,
-        # counted from the start of the sequence (0: all earlier keys); sink: fp32 [heads], one more term exp(sink) in each
-        # head's softmax denominator
+        # counted from the start of the sequence (0: all earlier keys)
         self.chunk_size = int(chunk_size)
-        self.sink = sink
 
     def forward(self, q, k, v, forward_batch: ForwardBatch, save_kv_cache: bool = True):
         return forward_batch.attn_backend.forward(q, k, v, self, forward_batch, save_kv_cache)

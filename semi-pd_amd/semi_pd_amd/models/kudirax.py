@@ -114,7 +114,7 @@ class KudiraxMixer(nn.Module):
         self.sink = nn.Parameter(torch.zeros(m.heads, dtype=torch.float32), requires_grad=False)
         self.vmix = nn.Parameter(torch.zeros((), dtype=dtype), requires_grad=False)
         self.attn = RadixAttention(m.heads, m.dim, m.scale, m.kv_heads, layer_id, logit_cap=m.softcap, v_head_dim=m.vdim,
-                                   chunk_size=m.chunk, sink=self.sink)
+                                   chunk_size=m.chunk)
 
     def forward(self, h: torch.Tensor, forward_batch, state: KudiraxForwardState) -> torch.Tensor:
         m = self.m
@@ -132,7 +132,7 @@ class KudiraxMixer(nn.Module):
                                    pool.get_value_buffer(lid), forward_batch.out_cache_loc, v_first=v_first,
                                    mix=self.vmix if v_first is not None else None)
         o = forward_batch.attn_backend.forward_local(p[:, : self.q_size], self.attn, forward_batch,
-                                                     gate=p[:, g_off: g_off + self.o_size])
+                                                     gate=p[:, g_off: g_off + self.o_size], sink=self.sink)
         return self.o_proj(o)
 
 

@@ -373,6 +373,18 @@ def test_minimal_sizes(dtype, tmp_path):
         assert _rel_err(got[n], K.forward(cfg, w, t)) < LIMIT[dtype], n
 
 
+def _check_generation(cfg, w, prompts, outs, steps):
+    exact = 0
+    for p, o in zip(prompts, outs):
+        assert len(o) == steps
+        logits = K.forward(cfg, w, p + o)
+        for i, tok in enumerate(o):
+            row = logits[len(p) + i - 1]
+            assert row[tok] >= row.max() - 0.08 * row.std(), (len(p), i)
+            exact += int(row.argmax().item() == tok)
+    assert exact > 0.9 * steps * len(prompts)
+
+
 def test_greedy_generation_through_the_engine(tmp_path):
     """Prompts of unequal length through Engine.generate (the unified scheduler: chunked prefill, decode graphs, sampler):
     every generated token is the plain model's argmax given the tokens before it, or within a small margin of it."""
@@ -389,12 +401,26 @@ def test_greedy_generation_through_the_engine(tmp_path):
         outs = eng.generate(prompts, SamplingParams(max_new_tokens=24, ignore_eos=True), timeout=300)
     finally:
         eng.shutdown()
-    exact = 0
-    for p, o in zip(prompts, outs):
-        assert len(o) == 24
-        logits = K.forward(cfg, w, p + o)
-        for i, tok in enumerate(o):
-            row = logits[len(p) + i - 1]
-            assert row[tok] >= row.max() - 0.08 * row.std(), (len(p), i)
-            exact += int(row.argmax().item() == tok)
-    assert exact > 0.9 * 24 * len(prompts)
+    _check_generation(cfg, w, prompts, outs, 24)
+
+
+def test_greedy_generation_through_the_semi_pd_engine(tmp_path):
+    """The same through a prefill and a decode process on one GPU: the per-layer pool regions and every parameter (the fp32
+    sinks, the blend weights) reach the prefill process through IPC handles; prompts are cut into 48-token portions there and
+    decoded in the other process."""
+    from semi_pd_amd.entrypoints.engine import Engine
+    from semi_pd_amd.managers.io_struct import SamplingParams
+    from semi_pd_amd.server_args import ServerArgs
+    cfg = CONFIGS["mixed"]
+    w = _write_checkpoint(str(tmp_path), cfg, seed=22)
+    prompts = [_tokens(n, cfg["vocab"], seed=100 + n) for n in (5, 90, 47, 130)]
+    sa = ServerArgs(model_path=str(tmp_path), load_format="auto", dtype="bfloat16", context_length=256, max_total_tokens=2048,
+                    max_running_requests=8, cuda_graph_max_bs=8, chunked_prefill_size=48, skip_tokenizer_init=True,
+                    enable_semi_pd=True, cu_mask_mode="env", prefill_cu_percent=50, decode_cu_percent=50, tune_prefill_gemm=False,
+                    watchdog_timeout=120.0)
+    eng = Engine(sa)
+    try:
+        outs = eng.generate(prompts, SamplingParams(max_new_tokens=16, ignore_eos=True), timeout=300)
+    finally:
+        eng.shutdown()
+    _check_generation(cfg, w, prompts, outs, 16)

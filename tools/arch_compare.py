@@ -1,0 +1,224 @@
+"""`python bench.py --arch-compare`: Kudirax next to the Llama-family model of equal size (random weights, one GPU).
+
+Two parts, printed as one JSON object:
+  * "models": prefill and decode throughput of a few-layer model of each design at layer sizes of real models, both driven
+    through the same replay scheduler (extend batches of whole prompts; decode batches through the captured graphs).
+  * "kernels": every kernel the design adds, alone, next to the kernel that does the like job for Llama, at the same
+    shape: time, achieved bytes/s or flop/s of the ALGORITHMIC work, the fraction of the roofline (8 TB/s, 2.5 PFLOP/s
+    dense bf16) and the ratio of the two fractions.
+"""
+from __future__ import annotations
+
+import json
+import math
+import time
+
+import torch
+
+HBM = 8.0e12
+MFMA = 2.5e15
+
+SIZES = {
+    # name: hidden, heads, kv heads, head size, ff, layers, vocab
+    "8b-layer": dict(hidden=4096, heads=32, kv=8, dim=128, ff=14336, layers=4, vocab=32000),
+    "3b-layer": dict(hidden=3072, heads=24, kv=8, dim=128, ff=8192, layers=4, vocab=32000),
+    "1b-layer": dict(hidden=2048, heads=32, kv=8, dim=64, ff=8192, layers=4, vocab=32000),
+}
+
+
+def _timed(fn, iters=20, warm=3):
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_time(e1) / iters * 1e-3
+
+
+def _configs(s, chunk):
+    from semi_pd_amd.models.kudirax import kudirax_uniform
+    from semi_pd_amd.models.llama import LlamaConfig
+    k = kudirax_uniform(s["vocab"], s["hidden"], s["layers"], s["heads"], s["kv"], s["dim"], s["dim"], s["ff"], chunk)
+    l = LlamaConfig(vocab_size=s["vocab"], hidden_size=s["hidden"], intermediate_size=s["ff"], num_hidden_layers=s["layers"],
+                    num_attention_heads=s["heads"], num_key_value_heads=s["kv"], head_dim=s["dim"],
+                    max_position_embeddings=16384)
+    return k, l
+
+
+def _model_throughput(cfg, prompt_len, prompts, decode_batch, decode_ctx, decode_steps):
+    from semi_pd_amd.managers.replay_scheduler import ReplayScheduler
+    from semi_pd_amd.model_executor.model_runner import ModelRunner
+    from semi_pd_amd.server_args import ServerArgs
+    ctx = max(prompt_len, decode_ctx + decode_steps + 8) + 8
+    total = max(prompt_len * prompts, decode_batch * (decode_ctx + decode_steps + 8)) + 64
+    sa = ServerArgs(model_config=cfg, load_format="dummy", context_length=ctx, max_total_tokens=total,
+                    max_running_requests=decode_batch, cuda_graph_max_bs=decode_batch, skip_tokenizer_init=True)
+    mr = ModelRunner(cfg, context_length=ctx, max_running_requests=decode_batch, max_total_tokens=total,
+                     cuda_graph_max_bs=decode_batch, mem_fraction_static=0.8)
+    mr.init_attention_backend()
+    mr.init_cuda_graphs()
+    sched = ReplayScheduler(sa, mr)
+    g = torch.Generator().manual_seed(0)
+
+    def toks(n):
+        return torch.randint(0, cfg.vocab_size, (n,), generator=g).tolist()
+
+    def prefill_once(tag):
+        ids = [f"{tag}{i}" for i in range(prompts)]
+        sched.replay_step([{"id": i, "tokens": toks(prompt_len), "want": [prompt_len - 1]} for i in ids], ids)
+
+    prefill_once("w")
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    reps = 3
+    for r in range(reps):
+        prefill_once(f"p{r}")
+    torch.cuda.synchronize()
+    prefill_tps = reps * prompts * prompt_len / (time.perf_counter() - t0)
+    # decode: requests of decode_ctx tokens (admitted four at a time), then single-token steps through the graphs
+    ids = [f"d{i}" for i in range(decode_batch)]
+    for a in range(0, decode_batch, 4):
+        sched.replay_step([{"id": i, "tokens": toks(decode_ctx), "want": []} for i in ids[a:a + 4]], [])
+    step = [{"id": i, "tokens": [1], "want": [0]} for i in ids]
+    for _ in range(3):
+        sched.replay_step(step, [])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(decode_steps):
+        sched.replay_step(step, [])
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    sched.replay_step([], ids)
+    out = {"prefill_tokens_per_s": round(prefill_tps), "decode_tokens_per_s": round(decode_steps * decode_batch / dt),
+           "decode_step_ms": round(dt / decode_steps * 1e3, 3)}
+    del sched, mr
+    torch.cuda.empty_cache()
+    return out
+
+
+def _kernel_pairs(s, chunk, dev):
+    """[(what, new kernel's record, like kernel's record)] at the layer shape `s`."""
+    from semi_pd_amd import ops
+    dt = torch.bfloat16
+    H, G, D, W, FF = s["heads"], s["kv"], s["dim"], s["hidden"], s["ff"]
+    E = D
+    out = []
+
+    def rec(t, nbytes=0.0, flops=0.0):
+        frac = max(nbytes / t / HBM, flops / t / MFMA)
+        return {"us": round(t * 1e6, 1), "TB_per_s": round(nbytes / t / 1e12, 2), "TFLOP_per_s": round(flops / t / 1e12, 1),
+                "of_roofline": round(frac, 3)}
+
+    # ---- prompt attention: 4 requests x 2048 new tokens ------------------------------------------------------------
+    B, L = 4, 2048
+    T = B * L
+    n_slots = T + 1
+    kp = torch.randn(n_slots, G, D, device=dev, dtype=dt)
+    vp = torch.randn(n_slots, G, E, device=dev, dtype=dt)
+    r2t = (torch.arange(T, device=dev, dtype=torch.int32) + 1).view(B, L).contiguous()
+    q = torch.randn(T, H * D, device=dev, dtype=dt)
+    o = torch.empty(T, H * E, device=dev, dtype=dt)
+    gate = torch.randn(T, H * E, device=dev, dtype=dt)
+    sink = torch.zeros(H, device=dev)
+    rows = torch.arange(B, device=dev)
+    lens = torch.full((B,), L, device=dev, dtype=torch.int64)
+    q_start = (torch.arange(B, device=dev, dtype=torch.int32) * L)
+    q_len = torch.full((B,), L, device=dev, dtype=torch.int32)
+    t_new = _timed(lambda: ops.local_attention_fwd(q, o, kp, vp, r2t, rows, lens, q_start, q_len, L, D ** -0.5, 30.0, chunk, sink, gate))
+    pairs_new = B * sum((p % chunk) + 1 for p in range(L)) if chunk else B * L * (L + 1) / 2
+    k_ext = torch.randn(T, G, D, device=dev, dtype=dt)
+    v_ext = torch.randn(T, G, D, device=dev, dtype=dt)
+    qo = (torch.arange(B + 1, device=dev, dtype=torch.int32) * L)
+    kvi = torch.zeros(B + 1, device=dev, dtype=torch.int32)
+    idx = torch.zeros(1, device=dev, dtype=torch.int32)
+    o3 = o.view(T, H, E)
+    t_old = _timed(lambda: ops.extend_attention_fwd(q.view(T, H, D), k_ext, v_ext, o3, kp, vp, qo, kvi, idx, None, None, L))
+    pairs_old = B * L * (L + 1) / 2
+    out.append((f"prompt attention, {B} x {L} tokens (new: blocks of {chunk})", rec(t_new, flops=2.0 * H * (D + E) * pairs_new),
+                rec(t_old, flops=2.0 * H * 2 * D * pairs_old)))
+    # ---- decode attention: 32 requests at 1100 tokens ----------------------------------------------------------------
+    B2, C = 32, 1100
+    n2 = B2 * C + 1
+    kp2 = torch.randn(n2, G, D, device=dev, dtype=dt)
+    vp2 = torch.randn(n2, G, E, device=dev, dtype=dt)
+    r2t2 = (torch.arange(B2 * C, device=dev, dtype=torch.int32) + 1).view(B2, C).contiguous()
+    q2 = torch.randn(B2, H * D, device=dev, dtype=dt)
+    o2 = torch.empty(B2, H * E, device=dev, dtype=dt)
+    g2 = torch.randn(B2, H * E, device=dev, dtype=dt)
+    rows2 = torch.arange(B2, device=dev)
+    lens2 = torch.full((B2,), C, device=dev, dtype=torch.int64)
+    t_new = _timed(lambda: ops.local_attention_fwd(q2, o2, kp2, vp2, r2t2, rows2, lens2, None, None, 1, D ** -0.5, 30.0, chunk, sink, g2))
+    keys_new = ((C - 1) % chunk) + 1 if chunk else C
+    from semi_pd_amd.layers.attention_backend import choose_kv_splits
+    splits = choose_kv_splits(B2, G, C, torch.cuda.get_device_properties(dev).multi_processor_count, 32)
+    logits = torch.empty(B2, H, splits, E + 1, device=dev, dtype=torch.float32)
+    indptr = (torch.arange(B2 + 1, device=dev, dtype=torch.int32) * C)
+    indices = r2t2.view(-1)
+    t_old = _timed(lambda: ops.decode_attention_fwd(q2.view(B2, H, D), kp2, vp2, o2.view(B2, H, E), indptr, indices, logits, splits, D ** -0.5))
+    out.append((f"decode attention, {B2} requests at {C} tokens (new: {keys_new} visible keys)",
+                rec(t_new, nbytes=B2 * G * (D + E) * 2.0 * keys_new), rec(t_old, nbytes=B2 * G * 2 * D * 2.0 * C)))
+    # ---- norm + residual -------------------------------------------------------------------------------------------
+    for Tn in (8192, 32):
+        y = torch.randn(Tn, W, device=dev, dtype=dt)
+        res = torch.randn(Tn, W, device=dev, dtype=torch.float32)
+        w = torch.ones(W, device=dev, dtype=dt)
+        b = torch.zeros(W, device=dev, dtype=dt)
+        t_new = _timed(lambda: ops.layernorm(y, w, b, 1e-5, residual=res, in_bias=b))
+        r16 = torch.randn(Tn, W, device=dev, dtype=dt)
+        t_old = _timed(lambda: ops.fused_add_rmsnorm(y, r16, w, 1e-5))
+        out.append((f"norm + residual add, {Tn} rows of {W}", rec(t_new, nbytes=Tn * W * (2 + 4 + 4 + 2.0)),
+                    rec(t_old, nbytes=Tn * W * 4 * 2.0)))
+    # ---- the step between the projection and the attention ---------------------------------------------------------------
+    Tn = 8192
+    cols = H * D + 2 * G * D + H * E
+    p = torch.randn(Tn, cols, device=dev, dtype=dt)
+    kp3 = torch.zeros(Tn + 1, G, D, device=dev, dtype=dt)
+    vp3 = torch.zeros(Tn + 1, G, E, device=dev, dtype=dt)
+    loc = torch.arange(1, Tn + 1, device=dev)
+    v0 = torch.randn(Tn, G * E, device=dev, dtype=dt)
+    mix = torch.tensor(0.5, device=dev, dtype=dt)
+    t_new = _timed(lambda: ops.unit_norm_and_store_kv(p, H, G, D, E, H * D, H * D + G * D, 1e-5, kp3, vp3, loc, v_first=v0, mix=mix))
+    from oracle import ops as O
+    cache = O.cos_sin_cache_from_inv_freq(O.rope_inv_freq(D, 10000.0), Tn + 1).to(dev)
+    qq = torch.randn(Tn, H * D, device=dev, dtype=dt)
+    kk = torch.randn(Tn, G * D, device=dev, dtype=dt)
+    vv = torch.randn(Tn, G * D, device=dev, dtype=dt)
+    pos = torch.arange(Tn, device=dev)
+    t_old = _timed(lambda: ops.rope_and_store_kv(pos, qq, kk, vv, D, cache, True, kp3, vp3, loc))
+    out.append((f"q / k preparation + KV-pool store, {Tn} tokens (new: unit norm + blend; like: rotation)",
+                rec(t_new, nbytes=Tn * 2.0 * (2 * H * D + 2 * G * D + 3 * G * E)), rec(t_old, nbytes=Tn * 2.0 * (2 * H * D + 4 * G * D))))
+    # ---- activation --------------------------------------------------------------------------------------------------
+    u = torch.randn(Tn, FF, device=dev, dtype=dt)
+    bb = torch.zeros(FF, device=dev, dtype=dt)
+    t_new = _timed(lambda: ops.bias_relu_square_(u, bb))
+    gu = torch.randn(Tn, 2 * FF, device=dev, dtype=dt)
+    t_old = _timed(lambda: ops.silu_and_mul(gu))
+    out.append((f"activation, {Tn} rows of {FF} (new: bias + squared ReLU in place; like: SiLU * mul)",
+                rec(t_new, nbytes=Tn * FF * 2 * 2.0), rec(t_old, nbytes=Tn * FF * 3 * 2.0)))
+    return out
+
+
+def main(args) -> dict:
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    chunk = int(getattr(args, "arch_chunk", 1024) or 0)
+    names = [n for n in (getattr(args, "arch_sizes", "") or ",".join(SIZES)).split(",") if n]
+    result = {"what": "Kudirax next to Llama at equal layer sizes", "dtype": "bf16", "data": "synthetic", "block": chunk,
+              "models": {}, "kernels": {}}
+    for name in names:
+        s = SIZES[name]
+        result["kernels"][name] = [
+            {"kernel": what, "kudirax": new, "llama": old,
+             "roofline_fraction_ratio": round(new["of_roofline"] / max(old["of_roofline"], 1e-9), 2)}
+            for what, new, old in _kernel_pairs(s, chunk, dev)]
+        kcfg, lcfg = _configs(s, chunk)
+        result["models"][name] = {
+            "layers": s["layers"],
+            "kudirax": _model_throughput(kcfg, 2048, 4, 32, 1100, 20),
+            "llama": _model_throughput(lcfg, 2048, 4, 32, 1100, 20)}
+    print(json.dumps(result), flush=True)
+    return result
