@@ -43,6 +43,126 @@ __global__ void __launch_bounds__(256) layernorm_kernel(const TIn* __restrict__ 
   }
 }
 
+// The same with the row held in registers: 16-byte loads, one pass over memory.  width % 8 == 0 (fp32 input: % 4 is
+// implied), width <= 256 * 8 * NC; rows and pointers 16-byte aligned.
+template <typename T, typename TIn, int NC>
+__global__ void __launch_bounds__(256) layernorm_vec_kernel(const TIn* __restrict__ in, int64_t in_ld, const T* __restrict__ in_bias,
+                                                            const T* __restrict__ w, const T* __restrict__ b, float eps,
+                                                            float* __restrict__ residual, int64_t res_ld, T* __restrict__ out,
+                                                            int64_t out_ld, int64_t width) {
+  __shared__ float red[16];
+  const int64_t r = blockIdx.x;
+  const TIn* x = in + r * in_ld;
+  float v[NC][8];
+  float s = 0.f;
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int64_t i = ((int64_t)c * 256 + threadIdx.x) * 8;
+    if (i < width) {
+      if constexpr (sizeof(TIn) == 4) {
+        const float4 a = *reinterpret_cast<const float4*>(x + i), d = *reinterpret_cast<const float4*>(x + i + 4);
+        v[c][0] = a.x; v[c][1] = a.y; v[c][2] = a.z; v[c][3] = a.w; v[c][4] = d.x; v[c][5] = d.y; v[c][6] = d.z; v[c][7] = d.w;
+      } else {
+        const Vec16<TIn> a = load16(x + i);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[c][u] = Elem<TIn>::to_f(a.e[u]);
+      }
+      if (in_bias) {
+        if constexpr (sizeof(T) == 2) {
+          const Vec16<T> a = load16(in_bias + i);
+#pragma unroll
+          for (int u = 0; u < 8; ++u) v[c][u] += Elem<T>::to_f(a.e[u]);
+        } else {
+#pragma unroll
+          for (int u = 0; u < 8; ++u) v[c][u] += Elem<T>::to_f(in_bias[i + u]);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) s += v[c][u];
+    }
+  }
+  const float mean = block_sum(s, red) / (float)width;
+  float q = 0.f;
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int64_t i = ((int64_t)c * 256 + threadIdx.x) * 8;
+    if (i < width) {
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const float d = v[c][u] - mean;
+        q += d * d;
+      }
+    }
+  }
+  __syncthreads();
+  const float var = block_sum(q, red) / (float)width;
+  const float rs = 1.0f / sqrtf(var + eps);
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int64_t i = ((int64_t)c * 256 + threadIdx.x) * 8;
+    if (i < width) {
+      float y[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) y[u] = (v[c][u] - mean) * rs * Elem<T>::to_f(w[i + u]) + Elem<T>::to_f(b[i + u]);
+      if (residual) {
+        float* rp = residual + r * res_ld + i;
+        float4 a = *reinterpret_cast<float4*>(rp), d = *reinterpret_cast<float4*>(rp + 4);
+        y[0] += a.x; y[1] += a.y; y[2] += a.z; y[3] += a.w; y[4] += d.x; y[5] += d.y; y[6] += d.z; y[7] += d.w;
+        a = float4{y[0], y[1], y[2], y[3]};
+        d = float4{y[4], y[5], y[6], y[7]};
+        *reinterpret_cast<float4*>(rp) = a;
+        *reinterpret_cast<float4*>(rp + 4) = d;
+      }
+      if (out) {
+        T* op = out + r * out_ld + i;
+        if constexpr (sizeof(T) == 2) {
+          Vec16<T> o;
+#pragma unroll
+          for (int u = 0; u < 8; ++u) o.e[u] = Elem<T>::from_f(y[u]);
+          store16(op, o);
+        } else {
+#pragma unroll
+          for (int u = 0; u < 8; ++u) op[u] = Elem<T>::from_f(y[u]);
+        }
+      }
+    }
+  }
+}
+
+// 8 elements per thread and step, 16-byte accesses (width % 8 == 0, rows 16-byte aligned)
+template <typename T>
+__global__ void __launch_bounds__(256) bias_relu_square_vec_kernel(T* __restrict__ u, int64_t ld, const T* __restrict__ bias,
+                                                                   int64_t rows, int64_t width) {
+  const int64_t per_row = width >> 3, n = rows * per_row;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / per_row, c = (i - r * per_row) << 3;
+    T* p = u + r * ld + c;
+    float v[8];
+    if constexpr (sizeof(T) == 2) {
+      const Vec16<T> a = load16(p);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[k] = Elem<T>::to_f(a.e[k]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[k] = Elem<T>::to_f(p[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      if (bias) v[k] += Elem<T>::to_f(bias[c + k]);
+      v[k] = v[k] > 0.f ? v[k] * v[k] : 0.f;
+    }
+    if constexpr (sizeof(T) == 2) {
+      Vec16<T> o;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) o.e[k] = Elem<T>::from_f(v[k]);
+      store16(p, o);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) p[k] = Elem<T>::from_f(v[k]);
+    }
+  }
+}
+
 template <typename T>
 __global__ void __launch_bounds__(256) bias_relu_square_kernel(T* __restrict__ u, int64_t ld, const T* __restrict__ bias,
                                                                int64_t rows, int64_t width) {
@@ -66,6 +186,32 @@ extern "C" int semipd_layernorm(const void* in, int64_t in_ld, int in_is_f32, co
   SEMIPD_CHECK_ARG(rows >= 0 && width > 0, SEMIPD_EINVAL, "layernorm: bad sizes");
   if (rows == 0) return 0;
   SEMIPD_CHECK_ARG(in && weight && bias && (residual || out), SEMIPD_EINVAL, "layernorm: null pointer");
+  const int64_t esz = dtype == SEMIPD_F32 ? 4 : 2, in_esz = in_is_f32 ? 4 : esz;
+  const bool vec = width % 8 == 0 && width <= 256 * 8 * 4 && aligned16(in) && (in_ld * in_esz) % 16 == 0 &&
+                   (!in_bias || aligned16(in_bias)) && (!residual || (aligned16(residual) && residual_ld % 4 == 0)) &&
+                   (!out || (aligned16(out) && (out_ld * esz) % 16 == 0));
+  if (vec) {
+    const bool two = width <= 256 * 8 * 2;
+    SEMIPD_DISPATCH_DTYPE(dtype, T, {
+      if (in_is_f32 && two)
+        hipLaunchKernelGGL((layernorm_vec_kernel<T, float, 2>), dim3((unsigned)rows), dim3(256), 0, as_stream(stream),
+                           (const float*)in, in_ld, (const T*)in_bias, (const T*)weight, (const T*)bias, eps, residual, residual_ld,
+                           (T*)out, out_ld, width);
+      else if (in_is_f32)
+        hipLaunchKernelGGL((layernorm_vec_kernel<T, float, 4>), dim3((unsigned)rows), dim3(256), 0, as_stream(stream),
+                           (const float*)in, in_ld, (const T*)in_bias, (const T*)weight, (const T*)bias, eps, residual, residual_ld,
+                           (T*)out, out_ld, width);
+      else if (two)
+        hipLaunchKernelGGL((layernorm_vec_kernel<T, T, 2>), dim3((unsigned)rows), dim3(256), 0, as_stream(stream), (const T*)in,
+                           in_ld, (const T*)in_bias, (const T*)weight, (const T*)bias, eps, residual, residual_ld, (T*)out, out_ld,
+                           width);
+      else
+        hipLaunchKernelGGL((layernorm_vec_kernel<T, T, 4>), dim3((unsigned)rows), dim3(256), 0, as_stream(stream), (const T*)in,
+                           in_ld, (const T*)in_bias, (const T*)weight, (const T*)bias, eps, residual, residual_ld, (T*)out, out_ld,
+                           width);
+    });
+    return launch_status("layernorm");
+  }
   SEMIPD_DISPATCH_DTYPE(dtype, T, {
     if (in_is_f32)
       hipLaunchKernelGGL((layernorm_kernel<T, float>), dim3((unsigned)rows), dim3(256), 0, as_stream(stream), (const float*)in,
@@ -84,6 +230,15 @@ extern "C" int semipd_bias_relu_square(void* u, int64_t ld, const void* bias, in
   if (rows == 0) return 0;
   SEMIPD_CHECK_ARG(u, SEMIPD_EINVAL, "bias_relu_square: null pointer");
   const int64_t n = rows * width;
+  const int64_t esz = dtype == SEMIPD_F32 ? 4 : 2;
+  if (width % 8 == 0 && aligned16(u) && (ld * esz) % 16 == 0) {
+    const int64_t nv = n / 8;
+    const unsigned vblocks = (unsigned)((nv + 255) / 256 < 16384 ? (nv + 255) / 256 : 16384);
+    SEMIPD_DISPATCH_DTYPE(dtype, T,
+                          hipLaunchKernelGGL((bias_relu_square_vec_kernel<T>), dim3(vblocks), dim3(256), 0, as_stream(stream),
+                                             (T*)u, ld, (const T*)bias, rows, width));
+    return launch_status("bias_relu_square");
+  }
   const unsigned blocks = (unsigned)((n + 255) / 256 < 8192 ? (n + 255) / 256 : 8192);
   SEMIPD_DISPATCH_DTYPE(dtype, T,
                         hipLaunchKernelGGL((bias_relu_square_kernel<T>), dim3(blocks), dim3(256), 0, as_stream(stream), (T*)u, ld,

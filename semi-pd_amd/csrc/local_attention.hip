@@ -9,7 +9,8 @@
 //    (chunk 0: lo = 0).  score = cap * tanh(scale * q.k / cap) (cap 0: none); the softmax denominator holds one more
 //    term exp(sink[head]) that has no value row.  Optional epilogue: out *= sigmoid(gate).
 //  * local_attention_mfma_kernel (bf16 / f16, head sizes in steps of 32 / 16): 64 query rows of one request and head
-//    per workgroup, S^T = K Q^T and O^T += V^T P^T on v_mfma_f32_16x16x32, P^T taken from the accumulators in place.
+//    per workgroup, S^T = K Q^T and O^T += V^T P^T on v_mfma_f32_16x16x32, P^T taken from the accumulators in place, V^T
+//    through transposing reads of a row-major LDS tile, the next step's loads in flight during the current one.
 //  * local_attention_decode_kernel (bf16 / f16): one workgroup per (request, kv head); the waves split the visible keys,
 //    the q heads of the group are the MFMA's columns, partials meet in LDS.
 #include "common.h"
@@ -53,6 +54,57 @@ __global__ void __launch_bounds__(256) unit_norm_kv_store_kernel(
         dst[e] = Elem<T>::from_f((1.0f - a) * Elem<T>::to_f(src[e]) + a * Elem<T>::to_f(v0[e]));
     } else {
       for (int e = lane; e < E; e += 64) dst[e] = src[e];
+    }
+  }
+}
+
+// The same for 16-bit types with 16-byte accesses: a head is taken by L = D / 8 lanes (a power of two), 64 / L heads per wave.
+template <typename T, int L>
+__global__ void __launch_bounds__(256) unit_norm_kv_store_vec_kernel(
+    T* __restrict__ qkv, int64_t ld, int64_t num_tokens, int H, int G, int D, int E, int64_t k_off, int64_t v_off, float eps,
+    const T* __restrict__ v_first, int64_t v_first_ld, const T* __restrict__ mix, T* __restrict__ k_pool,
+    T* __restrict__ v_pool, const int64_t* __restrict__ loc) {
+  constexpr int PER_WAVE = 64 / L;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, sl = lane % L;
+  const int items = H + 2 * G;
+  const int64_t item = ((int64_t)blockIdx.x * 4 + wave) * PER_WAVE + lane / L;
+  const bool on = item < num_tokens * items;
+  const int64_t t = on ? item / items : 0;
+  const int h = on ? (int)(item % items) : 0;
+  T* row = qkv + t * ld;
+  if (h < H + G) {               // (lanes of finished items still take part in the shuffles)
+    const bool is_q = h < H;
+    T* src = (is_q ? row + (int64_t)h * D : row + k_off + (int64_t)(h - H) * D) + sl * 8;
+    const Vec16<T> x = load16(src);
+    float f[8], ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      f[u] = Elem<T>::to_f(x.e[u]);
+      ss += f[u] * f[u];
+    }
+#pragma unroll
+    for (int o = L / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+    if (!on) return;
+    const float r = 1.0f / sqrtf(ss / (float)D + eps);
+    Vec16<T> y;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) y.e[u] = Elem<T>::from_f(f[u] * r);
+    store16(is_q ? src : k_pool + (loc[t] * G + (h - H)) * D + sl * 8, y);
+  } else {
+    if (!on) return;
+    const int g = h - H - G;
+    const T* src = row + v_off + (int64_t)g * E;
+    T* dst = v_pool + (loc[t] * G + g) * E;
+    const float a = v_first ? Elem<T>::to_f(mix[0]) : 0.f;
+    const T* v0 = v_first ? v_first + t * v_first_ld + (int64_t)g * E : nullptr;
+    for (int e = sl * 8; e < E; e += L * 8) {
+      Vec16<T> x = load16(src + e);
+      if (v0) {
+        const Vec16<T> z = load16(v0 + e);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) x.e[u] = Elem<T>::from_f((1.0f - a) * Elem<T>::to_f(x.e[u]) + a * Elem<T>::to_f(z.e[u]));
+      }
+      store16(dst + e, x);
     }
   }
 }
@@ -173,11 +225,12 @@ __global__ void __launch_bounds__(256) local_attention_rows_kernel(LocalAttnArgs
 
 // ------------------------------------------------------------------------------------------------ matrix-core forms
 // v_mfma_f32_16x16x32 (lane l: r = l & 15, g = l >> 4): a = A[row r][k 8g .. 8g+7], b = B[k 8g .. 8g+7][col r],
-// d[i] = D[row 4g + i][col r].  One step covers 32 keys: S^T = K Q^T is taken in two 16-row groups whose row rho stands
-// for key 8 (rho / 4) + rho % 4 (group A) and that key + 4 (group B), so that lane (r, g) ends up with the scores of keys
-// 8g .. 8g+7 of query r -- which is the b operand of O^T += V^T P^T as it stands.  V^T comes from an LDS tile [E][32].
+// d[i] = D[row 4g + i][col r].  One step covers 32 keys: S^T = K Q^T in two 16-row groups (keys 0 .. 15 and 16 .. 31 of the
+// step), so lane (r, g) ends with the scores of keys 4g .. 4g+3 and 16 + 4g .. + 3 of query r, which IS the b operand of
+// O^T += V^T P^T once the a operand numbers its k slots the same way: V^T comes out of a row-major LDS tile [32][E] through
+// the transposing read ds_read_b64_tr_b16, four keys x 16 value elements per 16-lane group.
+// The loads of step i + 1 (K fragments, V rows) are in flight in registers while step i is multiplied.
 typedef float f32x4 __attribute__((ext_vector_type(4)));
-constexpr int kVtLd = 40;                     // elements per V^T row in LDS: 32 keys + 8 of padding (80 bytes)
 
 template <typename T> __device__ __forceinline__ f32x4 mma16(const Frag16& a, const Frag16& b, f32x4 c);
 template <> __device__ __forceinline__ f32x4 mma16<bf16_t>(const Frag16& a, const Frag16& b, f32x4 c) {
@@ -196,98 +249,207 @@ __device__ __forceinline__ float fast_capped(float s, float scale, float cap) {
   return s;
 }
 
-// 32 rows of V (keys j0 .. j0+31 of the request, rows past `hi` as zeros) -> vt[e][key], by NT threads
-template <typename T, int NT>
-__device__ __forceinline__ void stage_vt(T* vt, const T* vp, const int32_t* row, int64_t j0, int64_t hi, int G, int gk, int E,
-                                         int tid) {
-  const int per_key = E >> 3;
-  for (int c = tid; c < 32 * per_key; c += NT) {
-    const int key = c / per_key, ec = c - key * per_key;
-    const int64_t j = j0 + key;
-    Vec16<T> v;
-    if (j <= hi) {
-      v = load16(vp + ((int64_t)row[j] * G + gk) * E + ec * 8);
-    } else {
-#pragma unroll
-      for (int u = 0; u < 8; ++u) v.e[u].v = 0;
-    }
-#pragma unroll
-    for (int u = 0; u < 8; ++u) vt[(ec * 8 + u) * kVtLd + key] = v.e[u];
-  }
-}
+// bytes per row of the V tile: E halves + padding so that the stride is 16 or 48 dwords mod 64 (conflict-free transposing
+// reads) and a multiple of 16 bytes
+__host__ __device__ inline int v_tile_row_bytes(int E) { return (E / 2 + (((16 - E / 2) % 32) + 32) % 32) * 4; }
+
+constexpr int kIdxLds = 2048;      // slots of the visible keys kept in LDS (8 KB): ranges up to this long
 
 template <int NE> struct SoftState {
   float m, l;
   f32x4 acc[NE];
 };
+template <int ND> struct KFrags {
+  Frag16 a[ND], b[ND];
+};
 
-// One step of 32 keys for the 16 columns of this wave.  sa / sb: the raw dot products of groups A and B (4 each) are
-// turned into probabilities against the running maximum, the accumulators are rescaled and V^T P^T is added.
-// ok(i): whether key 8g + i of the step is visible to this lane's column.
-template <typename T, int NE, typename Ok>
-__device__ __forceinline__ void soft_step(SoftState<NE>& st, f32x4 sa, f32x4 sb, float scale, float cap, Ok ok, const T* vt, int ne,
-                                          int r, int g) {
-  float s[8];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    s[i] = ok(i) ? fast_capped(sa[i], scale, cap) : -INFINITY;
-    s[4 + i] = ok(4 + i) ? fast_capped(sb[i], scale, cap) : -INFINITY;
-  }
-  float mt = s[0];
-#pragma unroll
-  for (int i = 1; i < 8; ++i) mt = fmaxf(mt, s[i]);
-  mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
-  mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-  const float m_new = fmaxf(st.m, mt);
-  const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-  const float alpha = __expf(st.m - m_safe);         // st.m = -inf: 0, and nothing has been accumulated yet
-  float p[8], sum = 0.f;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    p[i] = __expf(s[i] - m_safe);
-    sum += p[i];
-  }
-  st.l = st.l * alpha + sum;
-  st.m = m_new;
-  Frag16 pb;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) pb.w[i] = pack2<T>(p[2 * i], p[2 * i + 1]);
-#pragma unroll
-  for (int eb = 0; eb < NE; ++eb) {
-    if (eb < ne) {
-      Frag16 va;
-      va.u = *reinterpret_cast<const uint4*>(vt + (eb * 16 + r) * kVtLd + 8 * g);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) st.acc[eb][i] *= alpha;
-      st.acc[eb] = mma16<T>(va, pb, st.acc[eb]);
+// The walk over keys j_begin, j_begin + j_step, ... (steps of 32 keys, keys past j_end masked) for the 16 columns of this wave.
+//   NT threads (a workgroup with BLOCK_SYNC, else one wave) stage the V tile of every step; `tid` is the thread's index among
+//   them.  relevant(j0): whether this wave has anything to multiply in the step at j0 (it stages and syncs anyway).
+//   ok(j): whether key j is visible to this lane's column.
+//   BLOCK_SYNC (a workgroup walks together): the K rows of a step go through an LDS tile as well, loaded once for all waves
+//   in whole rows; a wave on its own takes its K fragments straight from the pool into operand layout.
+//   KS keys per step (32; the code also takes 64 = two halves between one pair of barriers, which measured slower: the
+//   staging registers of 64 rows push the 128 / 128 kernel into scratch at three waves per SIMD).
+template <typename T, int ND, int NE, int NT, bool BLOCK_SYNC, typename Ok, typename Relevant>
+__device__ __forceinline__ void key_walk(SoftState<NE>& st, const Frag16 (&qf)[ND], int nd, int ne, int E, const T* kp,
+                                         int64_t kstride, const T* vp, int64_t vstride, const int32_t* row, int64_t j_begin,
+                                         int64_t j_end, int64_t j_step, uint8_t* v_lds, int tid, float scale, float cap, Ok ok,
+                                         Relevant relevant, int r, int g, const int32_t* idx_lds, int64_t idx_base) {
+  constexpr int KS = 32;                          // keys per step
+  constexpr int NV = (NE * 2 * KS) / NT;          // 16-byte pieces of V per thread and step, at most
+  constexpr int NK = BLOCK_SYNC ? (ND * 4 * KS) / NT : 1;   // the same for K rows that go through LDS
+  const int per_key = E >> 3, pieces = KS * per_key, rs = v_tile_row_bytes(E);
+  const int per_key_k = nd * 4, pieces_k = KS * per_key_k, rsk = nd * 64 + 32;
+  uint8_t* k_lds = v_lds + KS * rs;
+  uint4 vr[NV];
+  uint4 kr[NK];
+  // pool slot of key j: from the copy of this part of the request's row in LDS when the caller made one (the load of a row
+  // of the pool then waits for nothing but itself), else from the table
+  auto slot_of = [&](int64_t j) -> int64_t { return idx_lds ? idx_lds[j - idx_base] : row[j]; };
+  auto sync = [&]() {
+    if constexpr (BLOCK_SYNC) {
+      __syncthreads();
+    } else {   // one wave: its LDS accesses execute in order; keep the compiler from reordering them
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
+  };
+  auto load_v = [&](int64_t j0) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int c = i * NT + tid;
+      if (c < pieces) {
+        const int key = c / per_key, ec = c - key * per_key;
+        const int64_t j = j0 + key;
+        vr[i] = j <= j_end ? *reinterpret_cast<const uint4*>(vp + slot_of(j) * vstride + ec * 8) : uint4{0u, 0u, 0u, 0u};
+      }
+    }
+  };
+  auto store_v = [&]() {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int c = i * NT + tid;
+      if (c < pieces) {
+        const int key = c / per_key, ec = c - key * per_key;
+        *reinterpret_cast<uint4*>(v_lds + key * rs + ec * 16) = vr[i];
+      }
+    }
+    if constexpr (BLOCK_SYNC) {
+#pragma unroll
+      for (int i = 0; i < NK; ++i) {
+        const int c = i * NT + tid;
+        if (c < pieces_k) {
+          const int key = c / per_key_k, ec = c - key * per_key_k;
+          *reinterpret_cast<uint4*>(k_lds + key * rsk + ec * 16) = kr[i];
+        }
+      }
+    }
+  };
+  auto load_k_rows = [&](int64_t j0) {
+#pragma unroll
+    for (int i = 0; i < NK; ++i) {
+      const int c = i * NT + tid;
+      if (c < pieces_k) {
+        const int key = c / per_key_k, ec = c - key * per_key_k;
+        const int64_t j = j0 + key;
+        kr[i] = j <= j_end ? *reinterpret_cast<const uint4*>(kp + slot_of(j) * kstride + ec * 8) : uint4{0u, 0u, 0u, 0u};
+      }
+    }
+  };
+  auto load_k = [&](int64_t j0, auto& k) {
+    const int64_t ja = j0 + r, jb = ja + 16;
+    const T* pa = kp + (ja <= j_end ? slot_of(ja) : 0) * kstride + 8 * g;
+    const T* pb = kp + (jb <= j_end ? slot_of(jb) : 0) * kstride + 8 * g;
+#pragma unroll
+    for (int kk = 0; kk < ND; ++kk)
+      if (kk < nd) {
+        k.a[kk].u = *reinterpret_cast<const uint4*>(pa + 32 * kk);
+        k.b[kk].u = *reinterpret_cast<const uint4*>(pb + 32 * kk);
+      }
+  };
+  auto compute = [&](int64_t j0, const auto& k, int half) {       // keys j0 .. j0 + 31 = rows 32 half .. of the tiles
+    f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (BLOCK_SYNC) {
+      const uint8_t* ra = k_lds + (32 * half + r) * rsk + g * 16;
+      const uint8_t* rb = ra + 16 * rsk;
+#pragma unroll
+      for (int kk = 0; kk < ND; ++kk)
+        if (kk < nd) {
+          Frag16 fa, fb;
+          fa.u = *reinterpret_cast<const uint4*>(ra + kk * 64);
+          fb.u = *reinterpret_cast<const uint4*>(rb + kk * 64);
+          sa = mma16<T>(fa, qf[kk], sa);
+          sb = mma16<T>(fb, qf[kk], sb);
+        }
+    } else {
+#pragma unroll
+      for (int kk = 0; kk < ND; ++kk)
+        if (kk < nd) {
+          sa = mma16<T>(k.a[kk], qf[kk], sa);
+          sb = mma16<T>(k.b[kk], qf[kk], sb);
+        }
+    }
+    float sc[8];
+    const int64_t ja = j0 + 4 * g, jb = ja + 16;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      sc[i] = ok(ja + i) ? fast_capped(sa[i], scale, cap) : -INFINITY;
+      sc[4 + i] = ok(jb + i) ? fast_capped(sb[i], scale, cap) : -INFINITY;
+    }
+    float mt = sc[0];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) mt = fmaxf(mt, sc[i]);
+    mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
+    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+    const float m_new = fmaxf(st.m, mt);
+    const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+    if (__any(m_new > st.m)) {
+      const float alpha = __expf(st.m - m_safe);       // st.m = -inf: 0, and nothing has been accumulated yet
+      st.l *= alpha;
+#pragma unroll
+      for (int eb = 0; eb < NE; ++eb)
+        if (eb < ne)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) st.acc[eb][i] *= alpha;
+      st.m = m_new;
+    }
+    float p[8], sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      p[i] = __expf(sc[i] - m_safe);
+      sum += p[i];
+    }
+    st.l += sum;
+    Frag16 pb;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) pb.w[i] = pack2<T>(p[2 * i], p[2 * i + 1]);
+    // 16-lane group g reads the 4 x 16 blocks {keys 4g .. 4g+3, then 16 + 4g ..} x {e = 16 eb .. + 15}: lane r of the group
+    // supplies row (r >> 2), columns 4 (r & 3) .. + 3 and receives column r
+    const uint8_t* vrow = v_lds + (32 * half + g * 4 + (r >> 2)) * rs + (r & 3) * 8;
+#pragma unroll
+    for (int eb = 0; eb < NE; ++eb)
+      if (eb < ne) {
+        Frag16 va;
+        va.s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vrow + eb * 32));
+        va.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vrow + 16 * rs + eb * 32));
+        st.acc[eb] = mma16<T>(va, pb, st.acc[eb]);
+      }
+  };
+  if (j_begin > j_end) return;
+  KFrags<BLOCK_SYNC ? 1 : ND> k0, k1;
+  load_v(j_begin);
+  if constexpr (BLOCK_SYNC) load_k_rows(j_begin);
+  else load_k(j_begin, k0);
+  auto step = [&](int64_t j0, auto& cur, auto& nxt) {
+    sync();                                            // the previous step's reads of the tiles are done
+    store_v();
+    sync();
+    const int64_t jn = j0 + j_step;
+    if (jn <= j_end) {                                 // in flight while this step is multiplied
+      load_v(jn);
+      if constexpr (BLOCK_SYNC) load_k_rows(jn);
+      else load_k(jn, nxt);
+    }
+    if (relevant(j0)) compute(j0, cur, 0);
+    if constexpr (KS == 64)
+      if (j0 + 32 <= j_end && relevant(j0 + 32)) compute(j0 + 32, cur, 1);
+  };
+  for (int64_t j0 = j_begin;;) {
+    step(j0, k0, k1);
+    j0 += j_step;
+    if (j0 > j_end) break;
+    step(j0, k1, k0);
+    j0 += j_step;
+    if (j0 > j_end) break;
   }
-}
-
-// the two groups of K rows of a step against the wave's Q fragments
-template <typename T, int ND>
-__device__ __forceinline__ void score_step(const Frag16 (&qf)[ND], int nd, const T* ka, const T* kb, int g, f32x4& sa, f32x4& sb) {
-  sa = f32x4{0.f, 0.f, 0.f, 0.f};
-  sb = f32x4{0.f, 0.f, 0.f, 0.f};
-  Frag16 fa[ND], fb[ND];
-#pragma unroll
-  for (int kk = 0; kk < ND; ++kk)
-    if (kk < nd) {
-      fa[kk].u = *reinterpret_cast<const uint4*>(ka + 32 * kk + 8 * g);
-      fb[kk].u = *reinterpret_cast<const uint4*>(kb + 32 * kk + 8 * g);
-    }
-#pragma unroll
-  for (int kk = 0; kk < ND; ++kk)
-    if (kk < nd) {
-      sa = mma16<T>(fa[kk], qf[kk], sa);
-      sb = mma16<T>(fb[kk], qf[kk], sb);
-    }
 }
 
 // Prompt portions: 64 query rows of one request and one head per workgroup, 16 per wave.
 template <typename T, int ND, int NE>
-__global__ void __launch_bounds__(256) local_attention_mfma_kernel(LocalAttnArgs a) {
-  __shared__ __attribute__((aligned(16))) T vt[NE * 16 * kVtLd];
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ND <= 4 ? 3 : 1))) local_attention_mfma_kernel(LocalAttnArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t v_lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
   const int h = blockIdx.y;
   // which request and which 64-row tile of it
@@ -295,14 +457,19 @@ __global__ void __launch_bounds__(256) local_attention_mfma_kernel(LocalAttnArgs
   int64_t q0 = 0;
   {
     int64_t left = blockIdx.x;
-    for (int rq = 0; rq < (int)a.batch; ++rq) {
-      const int64_t tiles = ((int64_t)a.q_len[rq] + 63) >> 6;
-      if (left < tiles) {
-        b = rq;
-        q0 = left << 6;
-        break;
+    for (int rq0 = 0; rq0 < (int)a.batch && b < 0; rq0 += 8) {     // eight lengths per round trip
+      int32_t n[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) n[u] = rq0 + u < (int)a.batch ? a.q_len[rq0 + u] : 0;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int64_t tiles = ((int64_t)n[u] + 63) >> 6;
+        if (b < 0 && left < tiles) {
+          b = rq0 + u;
+          q0 = left << 6;
+        }
+        if (b < 0) left -= tiles;
       }
-      left -= tiles;
     }
   }
   if (b < 0) return;
@@ -334,27 +501,17 @@ __global__ void __launch_bounds__(256) local_attention_mfma_kernel(LocalAttnArgs
 #pragma unroll
   for (int eb = 0; eb < NE; ++eb) st.acc[eb] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int32_t* row = a.req_to_token + a.req_pool_indices[b] * a.r2t_stride;
-  const T* kp = (const T*)a.k_pool + (int64_t)gk * D;
-  const T* vp = (const T*)a.v_pool;
-  const int64_t kstride = (int64_t)G * D;
-  const int ka_off = 8 * (r >> 2) + (r & 3);
-  for (int64_t j0 = blk_lo; j0 <= blk_hi; j0 += 32) {
-    __syncthreads();                                   // everyone is done with the previous V^T tile
-    stage_vt<T, 256>(vt, vp, row, j0, blk_hi, G, gk, E, tid);
+  __shared__ int32_t idx_lds[kIdxLds];
+  const bool idx_fits = blk_hi - blk_lo < kIdxLds;
+  if (idx_fits) {
+    for (int64_t j = blk_lo + tid; j <= blk_hi; j += 256) idx_lds[j - blk_lo] = row[j];
     __syncthreads();
-    if (!wave_on || j0 + 31 < w_lo || j0 > w_hi) continue;
-    const int64_t ja = j0 + ka_off, jb = ja + 4;
-    const T* ka = kp + (int64_t)(ja <= blk_hi ? row[ja] : 0) * kstride;
-    const T* kb = kp + (int64_t)(jb <= blk_hi ? row[jb] : 0) * kstride;
-    f32x4 sa, sb;
-    score_step<T, ND>(qf, nd, ka, kb, g, sa, sb);
-    const int64_t jl = j0 + 8 * g;
-    soft_step<T, NE>(st, sa, sb, a.scale, a.cap,
-                     [&](int i) { const int64_t j = jl + i; return q_ok && j >= my_lo && j <= my_pos; }, vt, ne, r, g);
   }
-  if (!q_ok) {
-    // (rows past the request's end took part in the shuffles above only)
-  }
+  key_walk<T, ND, NE, 256, true>(
+      st, qf, nd, ne, E, (const T*)a.k_pool + (int64_t)gk * D, (int64_t)G * D, (const T*)a.v_pool + (int64_t)gk * E,
+      (int64_t)G * E, row, blk_lo, blk_hi, 32, v_lds, tid, a.scale, a.cap,
+      [&](int64_t j) { return q_ok && j >= my_lo && j <= my_pos; },
+      [&](int64_t j0) { return wave_on && j0 + 31 >= w_lo && j0 <= w_hi; }, r, g, idx_fits ? idx_lds : nullptr, blk_lo);
   float l = st.l;
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
@@ -381,10 +538,10 @@ __global__ void __launch_bounds__(256) local_attention_mfma_kernel(LocalAttnArgs
 }
 
 // Decode steps: one workgroup per (request, kv head, group of 16 q heads); the q heads are the 16 columns, the four waves
-// take the 32-key steps in turn and meet in LDS.
+// take the 32-key steps in turn, each with a V tile of its own, and meet in LDS.
 template <typename T, int ND, int NE>
 __global__ void __launch_bounds__(256) local_attention_decode_kernel(LocalAttnArgs a) {
-  __shared__ __attribute__((aligned(16))) T vt[4][NE * 16 * kVtLd];
+  extern __shared__ __attribute__((aligned(16))) uint8_t v_lds[];
   __shared__ float part_ml[4][2][16];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
   const int b = blockIdx.x, gk = blockIdx.y;
@@ -410,25 +567,19 @@ __global__ void __launch_bounds__(256) local_attention_decode_kernel(LocalAttnAr
 #pragma unroll
   for (int eb = 0; eb < NE; ++eb) st.acc[eb] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int32_t* row = a.req_to_token + a.req_pool_indices[b] * a.r2t_stride;
-  const T* kp = (const T*)a.k_pool + (int64_t)gk * D;
-  const T* vp = (const T*)a.v_pool;
-  const int64_t kstride = (int64_t)G * D;
-  const int ka_off = 8 * (r >> 2) + (r & 3);
-  for (int64_t j0 = lo + 32 * wave; j0 <= pos; j0 += 128) {
-    // the wave's own V^T tile: its LDS accesses are executed in order, the barrier keeps the compiler from mixing them
-    __builtin_amdgcn_wave_barrier();
-    stage_vt<T, 64>(vt[wave], vp, row, j0, pos, G, gk, E, lane);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const int64_t ja = j0 + ka_off, jb = ja + 4;
-    const T* ka = kp + (int64_t)(ja <= pos ? row[ja] : 0) * kstride;
-    const T* kb = kp + (int64_t)(jb <= pos ? row[jb] : 0) * kstride;
-    f32x4 sa, sb;
-    score_step<T, ND>(qf, nd, ka, kb, g, sa, sb);
-    const int64_t jl = j0 + 8 * g;
-    soft_step<T, NE>(st, sa, sb, a.scale, a.cap, [&](int i) { return jl + i <= pos; }, vt[wave], ne, r, g);
+  // a wave's tile: 32 rows of the V tile, and room for its partial sums afterwards ([E][17] floats)
+  const int tile_bytes = 32 * v_tile_row_bytes(E) > E * 17 * 4 ? 32 * v_tile_row_bytes(E) : E * 17 * 4;
+  uint8_t* mine_b = v_lds + wave * tile_bytes;
+  __shared__ int32_t idx_lds[kIdxLds];
+  const bool idx_fits = pos - lo < kIdxLds;
+  if (idx_fits) {
+    for (int64_t j = lo + tid; j <= pos; j += 256) idx_lds[j - lo] = row[j];
+    __syncthreads();
   }
+  key_walk<T, ND, NE, 64, false>(
+      st, qf, nd, ne, E, (const T*)a.k_pool + (int64_t)gk * D, (int64_t)G * D, (const T*)a.v_pool + (int64_t)gk * E,
+      (int64_t)G * E, row, lo + 32 * wave, pos, 128, mine_b, lane, a.scale, a.cap, [&](int64_t j) { return j <= pos; },
+      [&](int64_t) { return true; }, r, g, idx_fits ? idx_lds : nullptr, lo);
   float l = st.l;
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
@@ -436,9 +587,10 @@ __global__ void __launch_bounds__(256) local_attention_decode_kernel(LocalAttnAr
     part_ml[wave][0][r] = st.m;
     part_ml[wave][1][r] = l;
   }
-  // a wave's partial sums go where its V^T tile was ([e][17] floats fit in [e][40] halves); only the wave itself read it
+  // a wave's partial sums go where its V tile was; only the wave itself read it
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
-  float* mine = reinterpret_cast<float*>(vt[wave]);
+  float* mine = reinterpret_cast<float*>(mine_b);
 #pragma unroll
   for (int eb = 0; eb < NE; ++eb)
     if (eb < ne)
@@ -466,7 +618,7 @@ __global__ void __launch_bounds__(256) local_attention_decode_kernel(LocalAttnAr
   for (int e = slice; e < E; e += 16) {
     float y = 0.f;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) y += f[w] * reinterpret_cast<const float*>(vt[w])[e * 17 + c];
+    for (int w = 0; w < 4; ++w) y += f[w] * reinterpret_cast<const float*>(v_lds + w * tile_bytes)[e * 17 + c];
     y *= inv;
     if (gt) y *= 1.0f / (1.0f + __expf(-Elem<T>::to_f(gt[e])));
     o[e] = Elem<T>::from_f(y);
@@ -495,6 +647,29 @@ extern "C" int semipd_unit_norm_kv_store(void* qkv, int64_t ld, int64_t num_toke
                        v_off >= k_off + (int64_t)num_kv_heads * qk_dim,
                    SEMIPD_EINVAL, "unit_norm_kv_store: column ranges overlap or leave the row");
   const int64_t items = num_tokens * (num_q_heads + 2 * num_kv_heads);
+  const int L = qk_dim / 8;
+  if ((dtype == SEMIPD_BF16 || dtype == SEMIPD_F16) && qk_dim % 8 == 0 && (L & (L - 1)) == 0 && L <= 64 && v_dim % 8 == 0 &&
+      ld % 8 == 0 && k_off % 8 == 0 && v_off % 8 == 0 && aligned16(qkv) && aligned16(k_pool) && aligned16(v_pool) &&
+      (!v_first || (aligned16(v_first) && v_first_ld % 8 == 0))) {
+    const int64_t per_block = 4 * (64 / L);
+    const unsigned vb = (unsigned)((items + per_block - 1) / per_block);
+#define SEMIPD_UNKS(LL)                                                                                                        \
+  SEMIPD_DISPATCH_HALF(dtype, T,                                                                                               \
+                       hipLaunchKernelGGL((unit_norm_kv_store_vec_kernel<T, LL>), dim3(vb), dim3(256), 0, as_stream(stream),     \
+                                          (T*)qkv, ld, num_tokens, num_q_heads, num_kv_heads, qk_dim, v_dim, k_off, v_off, eps,  \
+                                          (const T*)v_first, v_first_ld, (const T*)mix, (T*)k_pool, (T*)v_pool, loc))
+    switch (L) {
+      case 1: SEMIPD_UNKS(1); break;
+      case 2: SEMIPD_UNKS(2); break;
+      case 4: SEMIPD_UNKS(4); break;
+      case 8: SEMIPD_UNKS(8); break;
+      case 16: SEMIPD_UNKS(16); break;
+      case 32: SEMIPD_UNKS(32); break;
+      default: SEMIPD_UNKS(64); break;
+    }
+#undef SEMIPD_UNKS
+    return launch_status("unit_norm_kv_store");
+  }
   const unsigned blocks = (unsigned)((items + 3) / 4);
   SEMIPD_DISPATCH_DTYPE(dtype, T,
                         hipLaunchKernelGGL((unit_norm_kv_store_kernel<T>), dim3(blocks), dim3(256), 0, as_stream(stream),
@@ -530,24 +705,42 @@ extern "C" int semipd_local_attention(const void* q, int64_t q_ld, const void* g
   SEMIPD_CHECK_ARG(form != 2 || mfma_ok, SEMIPD_ESHAPE, "local_attention: the matrix-core forms do not take this shape or type");
   if (form != 1 && mfma_ok) {
     const bool small = qk_dim <= 128 && v_dim <= 128;
+    const int tile = 32 * v_tile_row_bytes(v_dim);                       // at most 32 * 576 bytes: below the 64 KB default
     if (q_start == nullptr || max_q_len <= 1) {
       const dim3 grid((unsigned)batch, (unsigned)num_kv_heads, (unsigned)((num_q_heads / num_kv_heads + 15) / 16));
+      const int merge = v_dim * 17 * 4;
+      const size_t lds = 4 * (size_t)(tile > merge ? tile : merge);      // at most 4 * 18 432 bytes: above the 64 KB default
+      if (lds > 65536) {
+        static std::atomic<uint64_t> done_bf16{0}, done_f16{0};
+        if (dtype == SEMIPD_BF16
+                ? ensure_dynamic_lds((const void*)local_attention_decode_kernel<bf16_t, 8, 16>, lds, done_bf16, "local_attention")
+                : ensure_dynamic_lds((const void*)local_attention_decode_kernel<f16_t, 8, 16>, lds, done_f16, "local_attention"))
+          return SEMIPD_EINVAL;
+      }
       if (dtype == SEMIPD_BF16) {
-        if (small) hipLaunchKernelGGL((local_attention_decode_kernel<bf16_t, 4, 8>), grid, dim3(256), 0, as_stream(stream), a);
-        else hipLaunchKernelGGL((local_attention_decode_kernel<bf16_t, 8, 16>), grid, dim3(256), 0, as_stream(stream), a);
+        if (small) hipLaunchKernelGGL((local_attention_decode_kernel<bf16_t, 4, 8>), grid, dim3(256), lds, as_stream(stream), a);
+        else hipLaunchKernelGGL((local_attention_decode_kernel<bf16_t, 8, 16>), grid, dim3(256), lds, as_stream(stream), a);
       } else {
-        if (small) hipLaunchKernelGGL((local_attention_decode_kernel<f16_t, 4, 8>), grid, dim3(256), 0, as_stream(stream), a);
-        else hipLaunchKernelGGL((local_attention_decode_kernel<f16_t, 8, 16>), grid, dim3(256), 0, as_stream(stream), a);
+        if (small) hipLaunchKernelGGL((local_attention_decode_kernel<f16_t, 4, 8>), grid, dim3(256), lds, as_stream(stream), a);
+        else hipLaunchKernelGGL((local_attention_decode_kernel<f16_t, 8, 16>), grid, dim3(256), lds, as_stream(stream), a);
       }
       return launch_status("local_attention_decode");
     }
     const dim3 grid((unsigned)((num_tokens + 63) / 64 + batch), (unsigned)num_q_heads);
+    const size_t tiles = (size_t)tile + 32 * (size_t)(qk_dim * 2 + 32);         // 32 V rows, then 32 K rows: at most 35.8 KB
+    if (tiles > 65536) {
+      static std::atomic<uint64_t> done_bf16{0}, done_f16{0};
+      if (dtype == SEMIPD_BF16
+              ? ensure_dynamic_lds((const void*)local_attention_mfma_kernel<bf16_t, 8, 16>, tiles, done_bf16, "local_attention")
+              : ensure_dynamic_lds((const void*)local_attention_mfma_kernel<f16_t, 8, 16>, tiles, done_f16, "local_attention"))
+        return SEMIPD_EINVAL;
+    }
     if (dtype == SEMIPD_BF16) {
-      if (small) hipLaunchKernelGGL((local_attention_mfma_kernel<bf16_t, 4, 8>), grid, dim3(256), 0, as_stream(stream), a);
-      else hipLaunchKernelGGL((local_attention_mfma_kernel<bf16_t, 8, 16>), grid, dim3(256), 0, as_stream(stream), a);
+      if (small) hipLaunchKernelGGL((local_attention_mfma_kernel<bf16_t, 4, 8>), grid, dim3(256), tiles, as_stream(stream), a);
+      else hipLaunchKernelGGL((local_attention_mfma_kernel<bf16_t, 8, 16>), grid, dim3(256), tiles, as_stream(stream), a);
     } else {
-      if (small) hipLaunchKernelGGL((local_attention_mfma_kernel<f16_t, 4, 8>), grid, dim3(256), 0, as_stream(stream), a);
-      else hipLaunchKernelGGL((local_attention_mfma_kernel<f16_t, 8, 16>), grid, dim3(256), 0, as_stream(stream), a);
+      if (small) hipLaunchKernelGGL((local_attention_mfma_kernel<f16_t, 4, 8>), grid, dim3(256), tiles, as_stream(stream), a);
+      else hipLaunchKernelGGL((local_attention_mfma_kernel<f16_t, 8, 16>), grid, dim3(256), tiles, as_stream(stream), a);
     }
     return launch_status("local_attention_mfma");
   }

@@ -141,7 +141,7 @@ def _kernel_pairs(s, chunk, dev):
     out.append((f"prompt attention, {B} x {L} tokens (new: blocks of {chunk})", rec(t_new, flops=2.0 * H * (D + E) * pairs_new),
                 rec(t_old, flops=2.0 * H * 2 * D * pairs_old)))
     # ---- decode attention: 32 requests at 1100 tokens ----------------------------------------------------------------
-    B2, C = 32, 1100
+    B2, C = 32, 1000
     n2 = B2 * C + 1
     kp2 = torch.randn(n2, G, D, device=dev, dtype=dt)
     vp2 = torch.randn(n2, G, E, device=dev, dtype=dt)
