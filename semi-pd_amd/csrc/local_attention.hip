@@ -123,6 +123,7 @@ struct LocalAttnArgs {
   const float* sink;
   float scale, cap;
   int chunk;
+  int64_t n_tiles;       // prompt form: 64-row tiles, an upper bound (tiles past the last request's do nothing)
 };
 
 __device__ __forceinline__ float capped(float s, float scale, float cap) {
@@ -349,7 +350,7 @@ __device__ __forceinline__ void key_walk(SoftState<NE>& st, const Frag16 (&qf)[N
         k.b[kk].u = *reinterpret_cast<const uint4*>(pb + 32 * kk);
       }
   };
-  auto compute = [&](int64_t j0, const auto& k, int half) {       // keys j0 .. j0 + 31 = rows 32 half .. of the tiles
+  auto compute = [&](int64_t j0, const auto& k, int half, auto after_scores) {   // keys j0 .. j0 + 31 = rows 32 half .. of the tiles
     f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
     if constexpr (BLOCK_SYNC) {
       const uint8_t* ra = k_lds + (32 * half + r) * rsk + g * 16;
@@ -371,6 +372,7 @@ __device__ __forceinline__ void key_walk(SoftState<NE>& st, const Frag16 (&qf)[N
           sb = mma16<T>(k.b[kk], qf[kk], sb);
         }
     }
+    after_scores();            // (a lone wave asks for the next step's K fragments here: the registers are free again)
     float sc[8];
     const int64_t ja = j0 + 4 * g, jb = ja + 16;
 #pragma unroll
@@ -418,7 +420,7 @@ __device__ __forceinline__ void key_walk(SoftState<NE>& st, const Frag16 (&qf)[N
       }
   };
   if (j_begin > j_end) return;
-  KFrags<BLOCK_SYNC ? 1 : ND> k0, k1;
+  KFrags<BLOCK_SYNC ? 1 : ND> k0;      // one set: a lone wave refills it as soon as the scores of a step are taken
   load_v(j_begin);
   if constexpr (BLOCK_SYNC) load_k_rows(j_begin);
   else load_k(j_begin, k0);
@@ -430,20 +432,18 @@ __device__ __forceinline__ void key_walk(SoftState<NE>& st, const Frag16 (&qf)[N
     if (jn <= j_end) {                                 // in flight while this step is multiplied
       load_v(jn);
       if constexpr (BLOCK_SYNC) load_k_rows(jn);
-      else load_k(jn, nxt);
     }
-    if (relevant(j0)) compute(j0, cur, 0);
-    if constexpr (KS == 64)
-      if (j0 + 32 <= j_end && relevant(j0 + 32)) compute(j0 + 32, cur, 1);
+    if constexpr (BLOCK_SYNC) {
+      if (relevant(j0)) compute(j0, cur, 0, [] {});
+      if constexpr (KS == 64)
+        if (j0 + 32 <= j_end && relevant(j0 + 32)) compute(j0 + 32, cur, 1, [] {});
+    } else {
+      compute(j0, cur, 0, [&] {
+        if (jn <= j_end) load_k(jn, nxt);
+      });
+    }
   };
-  for (int64_t j0 = j_begin;;) {
-    step(j0, k0, k1);
-    j0 += j_step;
-    if (j0 > j_end) break;
-    step(j0, k1, k0);
-    j0 += j_step;
-    if (j0 > j_end) break;
-  }
+  for (int64_t j0 = j_begin; j0 <= j_end; j0 += j_step) step(j0, k0, k0);
 }
 
 // Prompt portions: 64 query rows of one request and one head per workgroup, 16 per wave.
@@ -451,12 +451,24 @@ template <typename T, int ND, int NE>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ND <= 4 ? 3 : 1))) local_attention_mfma_kernel(LocalAttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t v_lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
-  const int h = blockIdx.y;
+  // Workgroup -> (kv head, 64-row tile, q head of the group), the last fastest.  Consecutive workgroup ids go round the
+  // eight XCDs, each with an L2 of its own; id L is therefore given work item (L % 8) * (N / 8) + L / 8, so that an XCD walks
+  // a CONTIGUOUS range of items: the q heads of a kv head and the neighbouring tiles of a block of positions -- which read the
+  // same K / V rows -- run next to each other on one L2 (N = gridDim.x, a multiple of 8).  (One workgroup per kv head and
+  // tile that takes the q heads in turn measured slower: a quarter of the workgroups, four times as long, fill the chip badly.)
+  const int64_t n_items = gridDim.x, item = (int64_t)(blockIdx.x & 7) * (n_items >> 3) + (blockIdx.x >> 3);
+  const int rep_h = a.H / a.G;
+  const int64_t n_tiles = a.n_tiles;
+  if (item >= n_tiles * a.H) return;
+  const int h = (int)(item / (n_tiles * rep_h)) * rep_h + (int)(item % rep_h);
+  // (tiles from the last to the first: the workgroups that start last are the first tiles of a block of positions, the ones
+  //  with the fewest keys, so the launch ends without a long tail)
+  const int64_t tile_id = n_tiles - 1 - (item / rep_h) % n_tiles;
   // which request and which 64-row tile of it
   int b = -1;
   int64_t q0 = 0;
   {
-    int64_t left = blockIdx.x;
+    int64_t left = tile_id;
     for (int rq0 = 0; rq0 < (int)a.batch && b < 0; rq0 += 8) {     // eight lengths per round trip
       int32_t n[8];
 #pragma unroll
@@ -537,12 +549,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ND <= 
     }
 }
 
-// Decode steps: one workgroup per (request, kv head, group of 16 q heads); the q heads are the 16 columns, the four waves
+// Decode steps: one workgroup per (request, kv head, group of 16 q heads); the q heads are the 16 columns, the waves
 // take the 32-key steps in turn, each with a V tile of its own, and meet in LDS.
-template <typename T, int ND, int NE>
-__global__ void __launch_bounds__(256) local_attention_decode_kernel(LocalAttnArgs a) {
+// (eight waves for head sizes up to 128, four above: the walk's registers at 256 / 256 do not fit eight waves per CU)
+template <typename T, int ND, int NE, int NW>
+__global__ void __launch_bounds__(64 * NW) local_attention_decode_kernel(LocalAttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t v_lds[];
-  __shared__ float part_ml[4][2][16];
+  __shared__ float part_ml[NW][2][16];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
   const int b = blockIdx.x, gk = blockIdx.y;
   const int D = a.D, E = a.E, G = a.G, nd = D >> 5, ne = E >> 4;
@@ -573,12 +586,12 @@ __global__ void __launch_bounds__(256) local_attention_decode_kernel(LocalAttnAr
   __shared__ int32_t idx_lds[kIdxLds];
   const bool idx_fits = pos - lo < kIdxLds;
   if (idx_fits) {
-    for (int64_t j = lo + tid; j <= pos; j += 256) idx_lds[j - lo] = row[j];
+    for (int64_t j = lo + tid; j <= pos; j += 64 * NW) idx_lds[j - lo] = row[j];
     __syncthreads();
   }
   key_walk<T, ND, NE, 64, false>(
       st, qf, nd, ne, E, (const T*)a.k_pool + (int64_t)gk * D, (int64_t)G * D, (const T*)a.v_pool + (int64_t)gk * E,
-      (int64_t)G * E, row, lo + 32 * wave, pos, 128, mine_b, lane, a.scale, a.cap, [&](int64_t j) { return j <= pos; },
+      (int64_t)G * E, row, lo + 32 * wave, pos, 32 * NW, mine_b, lane, a.scale, a.cap, [&](int64_t j) { return j <= pos; },
       [&](int64_t) { return true; }, r, g, idx_fits ? idx_lds : nullptr, lo);
   float l = st.l;
   l += __shfl_xor(l, 16, 64);
@@ -602,10 +615,10 @@ __global__ void __launch_bounds__(256) local_attention_decode_kernel(LocalAttnAr
   if (col0 + c >= rep) return;
   float m = -INFINITY;
 #pragma unroll
-  for (int w = 0; w < 4; ++w) m = fmaxf(m, part_ml[w][0][c]);
-  float f[4], lt = 0.f;
+  for (int w = 0; w < NW; ++w) m = fmaxf(m, part_ml[w][0][c]);
+  float f[NW], lt = 0.f;
 #pragma unroll
-  for (int w = 0; w < 4; ++w) {
+  for (int w = 0; w < NW; ++w) {
     const float mw = part_ml[w][0][c];
     f[w] = mw == -INFINITY ? 0.f : __expf(mw - m);
     lt += f[w] * part_ml[w][1][c];
@@ -615,10 +628,10 @@ __global__ void __launch_bounds__(256) local_attention_decode_kernel(LocalAttnAr
   const float inv = 1.0f / lt;
   T* o = (T*)a.out + t * a.out_ld + (int64_t)hh * E;
   const T* gt = a.gate ? (const T*)a.gate + t * a.gate_ld + (int64_t)hh * E : nullptr;
-  for (int e = slice; e < E; e += 16) {
+  for (int e = slice; e < E; e += 4 * NW) {
     float y = 0.f;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) y += f[w] * reinterpret_cast<const float*>(v_lds + w * tile_bytes)[e * 17 + c];
+    for (int w = 0; w < NW; ++w) y += f[w] * reinterpret_cast<const float*>(v_lds + w * tile_bytes)[e * 17 + c];
     y *= inv;
     if (gt) y *= 1.0f / (1.0f + __expf(-Elem<T>::to_f(gt[e])));
     o[e] = Elem<T>::from_f(y);
@@ -698,7 +711,7 @@ extern "C" int semipd_local_attention(const void* q, int64_t q_ld, const void* g
   SEMIPD_CHECK_ARG(chunk >= 0 && logit_cap >= 0.f, SEMIPD_EINVAL, "local_attention: bad chunk or cap");
   LocalAttnArgs a{q, q_ld, gate, gate_ld, out, out_ld, k_pool, v_pool, req_to_token, req_to_token_stride, req_pool_indices,
                   seq_lens, q_start, q_len, batch, num_tokens, num_q_heads, num_kv_heads, qk_dim, v_dim, sink, scale, logit_cap,
-                  chunk};
+                  chunk, 0};
   const bool half = dtype == SEMIPD_BF16 || dtype == SEMIPD_F16;
   const bool mfma_ok = half && local_mfma_shape_ok(qk_dim, v_dim) && aligned16(q) && q_ld % 8 == 0 && aligned16(k_pool) &&
                        aligned16(v_pool) && aligned16(out) && out_ld % 4 == 0;
@@ -709,24 +722,26 @@ extern "C" int semipd_local_attention(const void* q, int64_t q_ld, const void* g
     if (q_start == nullptr || max_q_len <= 1) {
       const dim3 grid((unsigned)batch, (unsigned)num_kv_heads, (unsigned)((num_q_heads / num_kv_heads + 15) / 16));
       const int merge = v_dim * 17 * 4;
-      const size_t lds = 4 * (size_t)(tile > merge ? tile : merge);      // at most 4 * 18 432 bytes: above the 64 KB default
+      const int nw = small ? 8 : 4;
+      const size_t lds = nw * (size_t)(tile > merge ? tile : merge);      // up to 80 KB: above the 64 KB default
       if (lds > 65536) {
-        static std::atomic<uint64_t> done_bf16{0}, done_f16{0};
-        if (dtype == SEMIPD_BF16
-                ? ensure_dynamic_lds((const void*)local_attention_decode_kernel<bf16_t, 8, 16>, lds, done_bf16, "local_attention")
-                : ensure_dynamic_lds((const void*)local_attention_decode_kernel<f16_t, 8, 16>, lds, done_f16, "local_attention"))
-          return SEMIPD_EINVAL;
+        static std::atomic<uint64_t> done[4] = {};
+        const void* fn = dtype == SEMIPD_BF16
+                             ? (small ? (const void*)local_attention_decode_kernel<bf16_t, 4, 8, 8> : (const void*)local_attention_decode_kernel<bf16_t, 8, 16, 4>)
+                             : (small ? (const void*)local_attention_decode_kernel<f16_t, 4, 8, 8> : (const void*)local_attention_decode_kernel<f16_t, 8, 16, 4>);
+        if (ensure_dynamic_lds(fn, lds, done[(dtype == SEMIPD_BF16 ? 0 : 2) + (small ? 0 : 1)], "local_attention")) return SEMIPD_EINVAL;
       }
       if (dtype == SEMIPD_BF16) {
-        if (small) hipLaunchKernelGGL((local_attention_decode_kernel<bf16_t, 4, 8>), grid, dim3(256), lds, as_stream(stream), a);
-        else hipLaunchKernelGGL((local_attention_decode_kernel<bf16_t, 8, 16>), grid, dim3(256), lds, as_stream(stream), a);
+        if (small) hipLaunchKernelGGL((local_attention_decode_kernel<bf16_t, 4, 8, 8>), grid, dim3(512), lds, as_stream(stream), a);
+        else hipLaunchKernelGGL((local_attention_decode_kernel<bf16_t, 8, 16, 4>), grid, dim3(256), lds, as_stream(stream), a);
       } else {
-        if (small) hipLaunchKernelGGL((local_attention_decode_kernel<f16_t, 4, 8>), grid, dim3(256), lds, as_stream(stream), a);
-        else hipLaunchKernelGGL((local_attention_decode_kernel<f16_t, 8, 16>), grid, dim3(256), lds, as_stream(stream), a);
+        if (small) hipLaunchKernelGGL((local_attention_decode_kernel<f16_t, 4, 8, 8>), grid, dim3(512), lds, as_stream(stream), a);
+        else hipLaunchKernelGGL((local_attention_decode_kernel<f16_t, 8, 16, 4>), grid, dim3(256), lds, as_stream(stream), a);
       }
       return launch_status("local_attention_decode");
     }
-    const dim3 grid((unsigned)((num_tokens + 63) / 64 + batch), (unsigned)num_q_heads);
+    a.n_tiles = (num_tokens + 63) / 64 + batch;
+    const dim3 grid((unsigned)((a.n_tiles * num_q_heads + 7) / 8 * 8));
     const size_t tiles = (size_t)tile + 32 * (size_t)(qk_dim * 2 + 32);         // 32 V rows, then 32 K rows: at most 35.8 KB
     if (tiles > 65536) {
       static std::atomic<uint64_t> done_bf16{0}, done_f16{0};
