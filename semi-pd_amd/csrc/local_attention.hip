@@ -241,14 +241,20 @@ template <> __device__ __forceinline__ f32x4 mma16<f16_t>(const Frag16& a, const
   return __builtin_amdgcn_mfma_f32_16x16x32_f16(a.f, b.f, c, 0, 0, 0);
 }
 
-__device__ __forceinline__ float fast_capped(float s, float scale, float cap) {
-  s *= scale;
-  if (cap > 0.f) {
-    const float e = __expf(2.0f * s / cap);   // tanh(x) = 1 - 2 / (exp(2x) + 1); exp overflow gives 1, underflow -1
-    s = cap * (1.0f - 2.0f / (e + 1.0f));
+// Scores live in the base-2 domain (multiplied by log2 e) so that every exponential is one v_exp_f32, and the cap is
+//   cap * tanh(x / cap) * log2e = A - 2 A / (exp2(c raw) + 1),  A = cap log2e,  c = 2 scale log2e / cap
+// (one exp, one reciprocal: exp2 overflow gives A, underflow -A).  Without a cap: raw * scale * log2e.
+constexpr float kLog2e = 1.4426950408889634f;
+struct ScoreMap {
+  float c, A;          // A == 0: no cap
+  __device__ __forceinline__ ScoreMap(float scale, float cap)
+      : c(cap > 0.f ? 2.0f * scale * kLog2e / cap : scale * kLog2e), A(cap > 0.f ? cap * kLog2e : 0.f) {}
+  __device__ __forceinline__ float operator()(float raw) const {
+    const float t = raw * c;
+    if (A == 0.f) return t;
+    return A - 2.0f * A * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(t) + 1.0f);
   }
-  return s;
-}
+};
 
 // bytes per row of the V tile: E halves + padding so that the stride is 16 or 48 dwords mod 64 (conflict-free transposing
 // reads) and a multiple of 16 bytes
@@ -285,6 +291,7 @@ __device__ __forceinline__ void key_walk(SoftState<NE>& st, const Frag16 (&qf)[N
   uint8_t* k_lds = v_lds + KS * rs;
   uint4 vr[NV];
   uint4 kr[NK];
+  const ScoreMap smap(scale, cap);
   // pool slot of key j: from the copy of this part of the request's row in LDS when the caller made one (the load of a row
   // of the pool then waits for nothing but itself), else from the table
   auto slot_of = [&](int64_t j) -> int64_t { return idx_lds ? idx_lds[j - idx_base] : row[j]; };
@@ -377,8 +384,8 @@ __device__ __forceinline__ void key_walk(SoftState<NE>& st, const Frag16 (&qf)[N
     const int64_t ja = j0 + 4 * g, jb = ja + 16;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      sc[i] = ok(ja + i) ? fast_capped(sa[i], scale, cap) : -INFINITY;
-      sc[4 + i] = ok(jb + i) ? fast_capped(sb[i], scale, cap) : -INFINITY;
+      sc[i] = ok(ja + i) ? smap(sa[i]) : -INFINITY;
+      sc[4 + i] = ok(jb + i) ? smap(sb[i]) : -INFINITY;
     }
     float mt = sc[0];
 #pragma unroll
@@ -388,7 +395,7 @@ __device__ __forceinline__ void key_walk(SoftState<NE>& st, const Frag16 (&qf)[N
     const float m_new = fmaxf(st.m, mt);
     const float m_safe = m_new == -INFINITY ? 0.f : m_new;
     if (__any(m_new > st.m)) {
-      const float alpha = __expf(st.m - m_safe);       // st.m = -inf: 0, and nothing has been accumulated yet
+      const float alpha = __builtin_amdgcn_exp2f(st.m - m_safe);   // st.m = -inf: 0, and nothing has been accumulated yet
       st.l *= alpha;
 #pragma unroll
       for (int eb = 0; eb < NE; ++eb)
@@ -400,7 +407,7 @@ __device__ __forceinline__ void key_walk(SoftState<NE>& st, const Frag16 (&qf)[N
     float p[8], sum = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      p[i] = __expf(sc[i] - m_safe);
+      p[i] = __builtin_amdgcn_exp2f(sc[i] - m_safe);
       sum += p[i];
     }
     st.l += sum;
@@ -448,7 +455,7 @@ __device__ __forceinline__ void key_walk(SoftState<NE>& st, const Frag16 (&qf)[N
 
 // Prompt portions: 64 query rows of one request and one head per workgroup, 16 per wave.
 template <typename T, int ND, int NE>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ND <= 4 ? 3 : 1))) local_attention_mfma_kernel(LocalAttnArgs a) {
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ND <= 4 ? 4 : 1))) local_attention_mfma_kernel(LocalAttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t v_lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
   // Workgroup -> (kv head, 64-row tile, q head of the group), the last fastest.  Consecutive workgroup ids go round the
@@ -528,7 +535,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ND <= 
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
   if (!q_ok) return;
-  if (a.sink != nullptr) l += __expf(a.sink[h] - st.m);
+  if (a.sink != nullptr) l += __builtin_amdgcn_exp2f(a.sink[h] * kLog2e - st.m);      // (the running maximum is in the base-2 domain)
   const float inv = 1.0f / l;
   T* o = (T*)a.out + (t0 + my_q) * a.out_ld + (int64_t)h * E;
   const T* gt = a.gate ? (const T*)a.gate + (t0 + my_q) * a.gate_ld + (int64_t)h * E : nullptr;
@@ -540,7 +547,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ND <= 
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         y[i] = st.acc[eb][i] * inv;
-        if (gt) y[i] *= 1.0f / (1.0f + __expf(-Elem<T>::to_f(gt[e0 + i])));
+        if (gt) y[i] *= __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-kLog2e * Elem<T>::to_f(gt[e0 + i])));
       }
       uint2 w;
       w.x = pack2<T>(y[0], y[1]);
@@ -620,11 +627,11 @@ __global__ void __launch_bounds__(64 * NW) local_attention_decode_kernel(LocalAt
 #pragma unroll
   for (int w = 0; w < NW; ++w) {
     const float mw = part_ml[w][0][c];
-    f[w] = mw == -INFINITY ? 0.f : __expf(mw - m);
+    f[w] = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - m);
     lt += f[w] * part_ml[w][1][c];
   }
   const int hh = gk * rep + col0 + c;
-  if (a.sink != nullptr) lt += __expf(a.sink[hh] - m);
+  if (a.sink != nullptr) lt += __builtin_amdgcn_exp2f(a.sink[hh] * kLog2e - m);
   const float inv = 1.0f / lt;
   T* o = (T*)a.out + t * a.out_ld + (int64_t)hh * E;
   const T* gt = a.gate ? (const T*)a.gate + t * a.gate_ld + (int64_t)hh * E : nullptr;
@@ -633,7 +640,7 @@ __global__ void __launch_bounds__(64 * NW) local_attention_decode_kernel(LocalAt
 #pragma unroll
     for (int w = 0; w < NW; ++w) y += f[w] * reinterpret_cast<const float*>(v_lds + w * tile_bytes)[e * 17 + c];
     y *= inv;
-    if (gt) y *= 1.0f / (1.0f + __expf(-Elem<T>::to_f(gt[e])));
+    if (gt) y *= __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-kLog2e * Elem<T>::to_f(gt[e])));
     o[e] = Elem<T>::from_f(y);
   }
 }
