@@ -1,8 +1,8 @@
 """Kudirax: a post-norm decoder whose attention is local to blocks of positions and carries a sink term.
 
-Per layer, on an fp32 residual stream x (the sublayers read x itself, the norm sits on their OUTPUT):
+Per layer, on an fp32 residual stream x (a sublayer's input is x unnormalised; the norm is applied to what it RETURNS):
     x <- x + LayerNorm1(mixer(x));   x <- x + LayerNorm2(ff(x))   (a layer may have no ff)
-mixer: q, k, v and an output gate from ONE merged GEMM; q and k divided per head by their root mean square (no weight, no
+mixer: q, k, v and an output gate from ONE merged GEMM; q and k scaled per head to unit RMS (no weight, no
 rotation: positions enter only through the mask); v optionally blended with the values the first blending layer made for
 the same token; attention over the keys of the query's own block of `chunk` positions (counted from the start of the
 sequence) up to the query, scores scale * q.k capped by cap * tanh(. / cap), one extra term exp(sink[head]) in the softmax

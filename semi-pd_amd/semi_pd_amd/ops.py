@@ -1288,8 +1288,8 @@ def moe_grouped_gemm_fp8(a_q: torch.Tensor, a_s: torch.Tensor, w_q: torch.Tensor
 def unit_norm_and_store_kv(qkv: torch.Tensor, num_q_heads: int, num_kv_heads: int, qk_dim: int, v_dim: int, k_off: int,
                            v_off: int, eps: float, k_buffer: torch.Tensor, v_buffer: torch.Tensor, loc: torch.Tensor,
                            v_first: Optional[torch.Tensor] = None, mix: Optional[torch.Tensor] = None) -> None:
-    """Rows of `qkv` [T, >= v_off + G * v_dim] hold q | k | v at columns 0, k_off, v_off.  Per head q and k are divided by
-    their root mean square (eps inside the root, fp32): q in place, k into k_buffer[loc]; v -- blended as
+    """Rows of `qkv` [T, >= v_off + G * v_dim] hold q | k | v at columns 0, k_off, v_off.  Per head q and k are scaled to
+    unit RMS (x / sqrt(mean(x^2) + eps), fp32): q in place, k into k_buffer[loc]; v -- blended as
     (1 - mix) v + mix v_first where v_first [T, G * v_dim] is given -- into v_buffer[loc].  One launch
     (csrc/local_attention.hip)."""
     if qkv.dim() != 2 or qkv.stride(1) != 1:
