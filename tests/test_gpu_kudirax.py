@@ -151,6 +151,19 @@ def test_attention_far_key_and_sink(dtype, form):
         assert want[-1].abs().mean() > 0.5
 
 
+@pytest.mark.parametrize("decode", [False, True])
+def test_attention_more_keys_than_the_slot_copy_holds(decode):
+    """Over 2048 visible keys (no blocks, and blocks of 2304): the matrix-core forms then read the slots from the table
+    instead of their copy in LDS; the key at position 5 dominates the last query."""
+    def standout(pre, ext):
+        return [([pre + ext - 1], [(5, 4.0, 3.0)])]
+
+    for chunk in (0, 2304):
+        reqs = [(2499, 1), (2100, 1), (40, 1)] if decode else [(0, 2300), (2290, 3)]
+        got, want = _attention_case(2, 1, 32, 16, chunk, 25.0, torch.bfloat16, 2, reqs, seed=4, standout=standout, decode=decode)
+        torch.testing.assert_close(got, want, **TOL[torch.bfloat16])
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,D,E", [(4, 2, 64, 32), (3, 3, 40, 24), (2, 1, 96, 200)])
 def test_unit_norm_blend_and_store(dtype, H, G, D, E):
@@ -225,6 +238,11 @@ CONFIGS = {
     "minimal": {"architecture": "Kudirax", "vocab": 64, "width": 64, "norm": {"eps": 1e-6}, "layers": [
         {"type": "attention", "mixer": _mixer(1, 1, 64, 64, 1, 5.0, False), "mlp": {"kind": "dense", "ff": 64}},
         {"type": "attention", "mixer": _mixer(1, 1, 64, 64, 7, 5.0, True), "mlp": {"kind": "dense", "ff": 64}}]},
+    # nothing a multiple of 8: width, vocabulary, head sizes, feed-forward; no layer blends; a block longer than any prompt here
+    "awkward": {"architecture": "Kudirax", "vocab": 301, "width": 100, "norm": {"eps": 1e-4}, "layers": [
+        {"type": "attention", "mixer": _mixer(3, 1, 24, 20, 3, 7.0, False), "mlp": {"kind": "dense", "ff": 130}},
+        {"type": "attention", "mixer": _mixer(5, 5, 12, 36, 500, 50.0, False, scale=0.4), "mlp": None},
+        {"type": "attention", "mixer": _mixer(2, 1, 50, 6, 11, 3.0, False), "mlp": {"kind": "dense", "ff": 36}}]},
 }
 
 
@@ -369,6 +387,20 @@ def test_minimal_sizes(dtype, tmp_path):
     sched = _scheduler(str(tmp_path), dtype, max_tokens=128, graphs=False)
     prompts = {"x": _tokens(40, 64, 1), "y": _tokens(9, 64, 2)}
     got = _run_schedule(sched, prompts, [[("x", 7), ("y", 2)], [("x", 1), ("y", 1)], [("x", 1), ("y", 1)], [("x", 31), ("y", 5)]])
+    for n, t in prompts.items():
+        assert _rel_err(got[n], K.forward(cfg, w, t)) < LIMIT[dtype], n
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_awkward_sizes(dtype, tmp_path):
+    """Sizes that no vector path takes (width 100, value size 20, a vocabulary of 301): every kernel's plain form, the
+    library GEMMs at odd shapes, the decode graphs."""
+    cfg = CONFIGS["awkward"]
+    w = _write_checkpoint(str(tmp_path), cfg, seed=8)
+    sched = _scheduler(str(tmp_path), dtype, max_tokens=192)
+    prompts = {"x": _tokens(70, 301, 3), "y": _tokens(23, 301, 4), "z": _tokens(1, 301, 5)}
+    got = _run_schedule(sched, prompts, [[("x", 30), ("y", 2), ("z", 1)], [("x", 1), ("y", 1)], [("x", 1), ("y", 1)],
+                                         [("x", 37), ("y", 19)], [("x", 1)]])
     for n, t in prompts.items():
         assert _rel_err(got[n], K.forward(cfg, w, t)) < LIMIT[dtype], n
 
