@@ -55,6 +55,7 @@ class KudiraxConfig:
     norm_eps: float = 1e-5
     layers: List[KudiraxLayerConfig] = field(default_factory=list)
     architectures: tuple = ("Kudirax",)
+    supports_float32 = True       # every kernel of its path is templated on the element type (ServerArgs --dtype float32)
 
     @property
     def num_hidden_layers(self) -> int:

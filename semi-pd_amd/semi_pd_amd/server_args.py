@@ -137,6 +137,12 @@ class ServerArgs:
         if self.model_config is None and self.model_path:
             from semi_pd_amd.model_loader import load_hf_config
             self.model_config = load_hf_config(self.model_path)
+        if self.dtype == "float32" and self.model_config is not None \
+                and not getattr(self.model_config, "supports_float32", False):
+            # fp32 serving needs every kernel of the model's path in fp32: the attention, RoPE and GEMM kernels of the other
+            # families are 16-bit only
+            raise ValueError(f"--dtype float32 is not supported for {type(self.model_config).__name__} "
+                             "(its kernels run in bfloat16 / float16)")
         if self.tokenizer_path is None:
             self.tokenizer_path = self.model_path
         if self.served_model_name is None:

@@ -98,6 +98,21 @@ def test_plain_model_prefix_property_and_block_locality():
     torch.testing.assert_close(p[0], torch.tensor([[0.5, 0.0], [1 / 3, 1 / 3]]))
 
 
+def test_command_line_reads_the_folder_and_float32_is_for_models_that_have_it(tmp_path):
+    import argparse
+    from semi_pd_amd import server_args as SA
+    with open(tmp_path / "config.json", "w") as f:
+        json.dump(CFG, f)
+    ap = argparse.ArgumentParser()
+    SA.add_cli_args(ap)
+    sa = SA.from_cli_args(ap.parse_args(["--model-path", str(tmp_path), "--dtype", "float32", "--skip-tokenizer-init"]))
+    assert type(sa.model_config).__name__ == "KudiraxConfig" and sa.torch_dtype == torch.float32 and sa.load_format == "auto"
+    from semi_pd_amd.models.llama import LlamaConfig
+    with pytest.raises(ValueError):
+        SA.ServerArgs(model_config=LlamaConfig(), dtype="float32")
+    assert SA.ServerArgs(model_config=LlamaConfig(), dtype="bfloat16").torch_dtype == torch.bfloat16
+
+
 def test_replay_runner_refuses_without_a_device():
     from semi_pd_amd.entrypoints import trace_replay
     if torch.cuda.is_available():
