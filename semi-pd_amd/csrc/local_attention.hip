@@ -276,8 +276,8 @@ template <int ND> struct KFrags {
 //   ok(j): whether key j is visible to this lane's column.
 //   BLOCK_SYNC (a workgroup walks together): the K rows of a step go through an LDS tile as well, loaded once for all waves
 //   in whole rows; a wave on its own takes its K fragments straight from the pool into operand layout.
-//   KS keys per step (32; the code also takes 64 = two halves between one pair of barriers, which measured slower: the
-//   staging registers of 64 rows push the 128 / 128 kernel into scratch at three waves per SIMD).
+//   32 keys per step (64 between one pair of barriers measured slower: the staging registers of 64 rows push the 128 / 128
+//   kernel into scratch).
 template <typename T, int ND, int NE, int NT, bool BLOCK_SYNC, typename Ok, typename Relevant>
 __device__ __forceinline__ void key_walk(SoftState<NE>& st, const Frag16 (&qf)[ND], int nd, int ne, int E, const T* kp,
                                          int64_t kstride, const T* vp, int64_t vstride, const int32_t* row, int64_t j_begin,
@@ -288,10 +288,27 @@ __device__ __forceinline__ void key_walk(SoftState<NE>& st, const Frag16 (&qf)[N
   constexpr int NK = BLOCK_SYNC ? (ND * 4 * KS) / NT : 1;   // the same for K rows that go through LDS
   const int per_key = E >> 3, pieces = KS * per_key, rs = v_tile_row_bytes(E);
   const int per_key_k = nd * 4, pieces_k = KS * per_key_k, rsk = nd * 64 + 32;
+  // a workgroup keeps TWO pairs of tiles: while step i is multiplied out of one, the rows of step i + 1 land in the other,
+  // and one barrier per step separates them
+  const int tile_pair = KS * (rs + rsk);
   uint8_t* k_lds = v_lds + KS * rs;
   uint4 vr[NV];
   uint4 kr[NK];
   const ScoreMap smap(scale, cap);
+  // which row and which 16 bytes of it each of this thread's pieces is (the same in every step)
+  int v_key[NV], v_ec[NV], k_key[NK], k_ec[NK];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = i * NT + tid;
+    v_key[i] = c < pieces ? c / per_key : -1;
+    v_ec[i] = c < pieces ? c - v_key[i] * per_key : 0;
+  }
+#pragma unroll
+  for (int i = 0; i < NK; ++i) {
+    const int c = i * NT + tid;
+    k_key[i] = (BLOCK_SYNC && c < pieces_k) ? c / per_key_k : -1;
+    k_ec[i] = (BLOCK_SYNC && c < pieces_k) ? c - k_key[i] * per_key_k : 0;
+  }
   // pool slot of key j: from the copy of this part of the request's row in LDS when the caller made one (the load of a row
   // of the pool then waits for nothing but itself), else from the table
   auto slot_of = [&](int64_t j) -> int64_t { return idx_lds ? idx_lds[j - idx_base] : row[j]; };
@@ -306,45 +323,29 @@ __device__ __forceinline__ void key_walk(SoftState<NE>& st, const Frag16 (&qf)[N
   };
   auto load_v = [&](int64_t j0) {
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      const int c = i * NT + tid;
-      if (c < pieces) {
-        const int key = c / per_key, ec = c - key * per_key;
-        const int64_t j = j0 + key;
-        vr[i] = j <= j_end ? *reinterpret_cast<const uint4*>(vp + slot_of(j) * vstride + ec * 8) : uint4{0u, 0u, 0u, 0u};
+    for (int i = 0; i < NV; ++i)
+      if (v_key[i] >= 0) {
+        const int64_t j = j0 + v_key[i];
+        vr[i] = j <= j_end ? *reinterpret_cast<const uint4*>(vp + slot_of(j) * vstride + v_ec[i] * 8) : uint4{0u, 0u, 0u, 0u};
       }
-    }
   };
-  auto store_v = [&]() {
+  auto store_v = [&](int buf) {        // buf: which pair of tiles (a lone wave has one)
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      const int c = i * NT + tid;
-      if (c < pieces) {
-        const int key = c / per_key, ec = c - key * per_key;
-        *reinterpret_cast<uint4*>(v_lds + key * rs + ec * 16) = vr[i];
-      }
-    }
+    for (int i = 0; i < NV; ++i)
+      if (v_key[i] >= 0) *reinterpret_cast<uint4*>(v_lds + buf * tile_pair + v_key[i] * rs + v_ec[i] * 16) = vr[i];
     if constexpr (BLOCK_SYNC) {
 #pragma unroll
-      for (int i = 0; i < NK; ++i) {
-        const int c = i * NT + tid;
-        if (c < pieces_k) {
-          const int key = c / per_key_k, ec = c - key * per_key_k;
-          *reinterpret_cast<uint4*>(k_lds + key * rsk + ec * 16) = kr[i];
-        }
-      }
+      for (int i = 0; i < NK; ++i)
+        if (k_key[i] >= 0) *reinterpret_cast<uint4*>(k_lds + buf * tile_pair + k_key[i] * rsk + k_ec[i] * 16) = kr[i];
     }
   };
   auto load_k_rows = [&](int64_t j0) {
 #pragma unroll
-    for (int i = 0; i < NK; ++i) {
-      const int c = i * NT + tid;
-      if (c < pieces_k) {
-        const int key = c / per_key_k, ec = c - key * per_key_k;
-        const int64_t j = j0 + key;
-        kr[i] = j <= j_end ? *reinterpret_cast<const uint4*>(kp + slot_of(j) * kstride + ec * 8) : uint4{0u, 0u, 0u, 0u};
+    for (int i = 0; i < NK; ++i)
+      if (k_key[i] >= 0) {
+        const int64_t j = j0 + k_key[i];
+        kr[i] = j <= j_end ? *reinterpret_cast<const uint4*>(kp + slot_of(j) * kstride + k_ec[i] * 8) : uint4{0u, 0u, 0u, 0u};
       }
-    }
   };
   auto load_k = [&](int64_t j0, auto& k) {
     const int64_t ja = j0 + r, jb = ja + 16;
@@ -357,10 +358,10 @@ __device__ __forceinline__ void key_walk(SoftState<NE>& st, const Frag16 (&qf)[N
         k.b[kk].u = *reinterpret_cast<const uint4*>(pb + 32 * kk);
       }
   };
-  auto compute = [&](int64_t j0, const auto& k, int half, auto after_scores) {   // keys j0 .. j0 + 31 = rows 32 half .. of the tiles
+  auto compute = [&](int64_t j0, const auto& k, int half, auto after_scores) {   // keys j0 .. j0 + 31 out of tile pair `half`
     f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
     if constexpr (BLOCK_SYNC) {
-      const uint8_t* ra = k_lds + (32 * half + r) * rsk + g * 16;
+      const uint8_t* ra = k_lds + half * tile_pair + r * rsk + g * 16;
       const uint8_t* rb = ra + 16 * rsk;
 #pragma unroll
       for (int kk = 0; kk < ND; ++kk)
@@ -416,7 +417,7 @@ __device__ __forceinline__ void key_walk(SoftState<NE>& st, const Frag16 (&qf)[N
     for (int i = 0; i < 4; ++i) pb.w[i] = pack2<T>(p[2 * i], p[2 * i + 1]);
     // 16-lane group g reads the 4 x 16 blocks {keys 4g .. 4g+3, then 16 + 4g ..} x {e = 16 eb .. + 15}: lane r of the group
     // supplies row (r >> 2), columns 4 (r & 3) .. + 3 and receives column r
-    const uint8_t* vrow = v_lds + (32 * half + g * 4 + (r >> 2)) * rs + (r & 3) * 8;
+    const uint8_t* vrow = v_lds + half * tile_pair + (g * 4 + (r >> 2)) * rs + (r & 3) * 8;
 #pragma unroll
     for (int eb = 0; eb < NE; ++eb)
       if (eb < ne) {
@@ -431,26 +432,32 @@ __device__ __forceinline__ void key_walk(SoftState<NE>& st, const Frag16 (&qf)[N
   load_v(j_begin);
   if constexpr (BLOCK_SYNC) load_k_rows(j_begin);
   else load_k(j_begin, k0);
-  auto step = [&](int64_t j0, auto& cur, auto& nxt) {
-    sync();                                            // the previous step's reads of the tiles are done
-    store_v();
+  if constexpr (BLOCK_SYNC) {
+    store_v(0);
     sync();
-    const int64_t jn = j0 + j_step;
-    if (jn <= j_end) {                                 // in flight while this step is multiplied
-      load_v(jn);
-      if constexpr (BLOCK_SYNC) load_k_rows(jn);
+    int buf = 0;
+    for (int64_t j0 = j_begin; j0 <= j_end; j0 += j_step, buf ^= 1) {
+      const int64_t jn = j0 + j_step;
+      if (jn <= j_end) {                                 // in flight while this step is multiplied
+        load_v(jn);
+        load_k_rows(jn);
+      }
+      if (relevant(j0)) compute(j0, k0, buf, [] {});
+      if (jn <= j_end) store_v(buf ^ 1);
+      sync();       // the next step's rows are in place, and everyone is done with this step's
     }
-    if constexpr (BLOCK_SYNC) {
-      if (relevant(j0)) compute(j0, cur, 0, [] {});
-      if constexpr (KS == 64)
-        if (j0 + 32 <= j_end && relevant(j0 + 32)) compute(j0 + 32, cur, 1, [] {});
-    } else {
-      compute(j0, cur, 0, [&] {
-        if (jn <= j_end) load_k(jn, nxt);
+  } else {
+    for (int64_t j0 = j_begin; j0 <= j_end; j0 += j_step) {
+      const int64_t jn = j0 + j_step;
+      sync();                                            // the previous step's reads of the tile are done
+      store_v(0);
+      sync();
+      if (jn <= j_end) load_v(jn);                       // in flight while this step is multiplied
+      compute(j0, k0, 0, [&] {
+        if (jn <= j_end) load_k(jn, k0);
       });
     }
-  };
-  for (int64_t j0 = j_begin; j0 <= j_end; j0 += j_step) step(j0, k0, k0);
+  }
 }
 
 // Prompt portions: 64 query rows of one request and one head per workgroup, 16 per wave.
@@ -520,40 +527,49 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ND <= 
 #pragma unroll
   for (int eb = 0; eb < NE; ++eb) st.acc[eb] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int32_t* row = a.req_to_token + a.req_pool_indices[b] * a.r2t_stride;
-  __shared__ int32_t idx_lds[kIdxLds];
-  const bool idx_fits = blk_hi - blk_lo < kIdxLds;
-  if (idx_fits) {
-    for (int64_t j = blk_lo + tid; j <= blk_hi; j += 256) idx_lds[j - blk_lo] = row[j];
-    __syncthreads();
-  }
   key_walk<T, ND, NE, 256, true>(
       st, qf, nd, ne, E, (const T*)a.k_pool + (int64_t)gk * D, (int64_t)G * D, (const T*)a.v_pool + (int64_t)gk * E,
       (int64_t)G * E, row, blk_lo, blk_hi, 32, v_lds, tid, a.scale, a.cap,
       [&](int64_t j) { return q_ok && j >= my_lo && j <= my_pos; },
-      [&](int64_t j0) { return wave_on && j0 + 31 >= w_lo && j0 <= w_hi; }, r, g, idx_fits ? idx_lds : nullptr, blk_lo);
+      [&](int64_t j0) { return wave_on && j0 + 31 >= w_lo && j0 <= w_hi; }, r, g, nullptr, blk_lo);
   float l = st.l;
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
-  if (!q_ok) return;
+  if (!wave_on) return;
   if (a.sink != nullptr) l += __builtin_amdgcn_exp2f(a.sink[h] * kLog2e - st.m);      // (the running maximum is in the base-2 domain)
-  const float inv = 1.0f / l;
-  T* o = (T*)a.out + (t0 + my_q) * a.out_ld + (int64_t)h * E;
-  const T* gt = a.gate ? (const T*)a.gate + (t0 + my_q) * a.gate_ld + (int64_t)h * E : nullptr;
+  const float inv = q_ok ? 1.0f / l : 0.f;
+  // Epilogue through LDS (the tiles are free: the walk ends on a barrier): a lane holds 4 value elements of one row per
+  // 16-element block -- written out like that, rows would go to memory in 8-byte pieces; the wave lays its 16 x E tile down in
+  // LDS and takes it up again in whole 16-byte pieces of consecutive lanes, so the gate is read and the result written in
+  // full rows.
+  const int ors = E * 2 + 16;
+  uint8_t* o_lds = v_lds + wave * 16 * ors;
 #pragma unroll
   for (int eb = 0; eb < NE; ++eb)
     if (eb < ne) {
-      const int e0 = eb * 16 + 4 * g;
-      float y[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        y[i] = st.acc[eb][i] * inv;
-        if (gt) y[i] *= __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-kLog2e * Elem<T>::to_f(gt[e0 + i])));
-      }
       uint2 w;
-      w.x = pack2<T>(y[0], y[1]);
-      w.y = pack2<T>(y[2], y[3]);
-      *reinterpret_cast<uint2*>(o + e0) = w;
+      w.x = pack2<T>(st.acc[eb][0] * inv, st.acc[eb][1] * inv);
+      w.y = pack2<T>(st.acc[eb][2] * inv, st.acc[eb][3] * inv);
+      *reinterpret_cast<uint2*>(o_lds + r * ors + (eb * 16 + 4 * g) * 2) = w;
     }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  const int per_row = E >> 3;
+  for (int c = lane; c < 16 * per_row; c += 64) {
+    const int rr = c / per_row, ec = c - rr * per_row;
+    if (wq0 + rr >= qn) continue;
+    Vec16<T> v = *reinterpret_cast<const Vec16<T>*>(o_lds + rr * ors + ec * 16);
+    const int64_t t = t0 + wq0 + rr;
+    if (a.gate) {
+      const Vec16<T> gv = load16((const T*)a.gate + t * a.gate_ld + (int64_t)h * E + ec * 8);
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        v.e[u] = Elem<T>::from_f(Elem<T>::to_f(v.e[u]) *
+                                 __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-kLog2e * Elem<T>::to_f(gv.e[u]))));
+    }
+    store16((T*)a.out + t * a.out_ld + (int64_t)h * E + ec * 8, v);
+  }
 }
 
 // Decode steps: one workgroup per (request, kv head, group of 16 q heads); the q heads are the 16 columns, the waves
@@ -721,7 +737,8 @@ extern "C" int semipd_local_attention(const void* q, int64_t q_ld, const void* g
                   chunk, 0};
   const bool half = dtype == SEMIPD_BF16 || dtype == SEMIPD_F16;
   const bool mfma_ok = half && local_mfma_shape_ok(qk_dim, v_dim) && aligned16(q) && q_ld % 8 == 0 && aligned16(k_pool) &&
-                       aligned16(v_pool) && aligned16(out) && out_ld % 4 == 0;
+                       aligned16(v_pool) && aligned16(out) && out_ld % 8 == 0 &&
+                       (gate == nullptr || (aligned16(gate) && gate_ld % 8 == 0));
   SEMIPD_CHECK_ARG(form != 2 || mfma_ok, SEMIPD_ESHAPE, "local_attention: the matrix-core forms do not take this shape or type");
   if (form != 1 && mfma_ok) {
     const bool small = qk_dim <= 128 && v_dim <= 128;
@@ -749,7 +766,7 @@ extern "C" int semipd_local_attention(const void* q, int64_t q_ld, const void* g
     }
     a.n_tiles = (num_tokens + 63) / 64 + batch;
     const dim3 grid((unsigned)((a.n_tiles * num_q_heads + 7) / 8 * 8));
-    const size_t tiles = (size_t)tile + 32 * (size_t)(qk_dim * 2 + 32);         // 32 V rows, then 32 K rows: at most 35.8 KB
+    const size_t tiles = 2 * ((size_t)tile + 32 * (size_t)(qk_dim * 2 + 32));   // two pairs of (32 V rows, 32 K rows): at most 71.7 KB
     if (tiles > 65536) {
       static std::atomic<uint64_t> done_bf16{0}, done_f16{0};
       if (dtype == SEMIPD_BF16
