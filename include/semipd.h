@@ -811,6 +811,61 @@ int semipd_layernorm(const void* in, int64_t in_ld, int in_is_f32, const void* i
  * counterpart. */
 int semipd_bias_relu_square(void* u, int64_t ld, const void* bias, int64_t rows, int64_t width, int dtype, void* stream);
 
+/* ------------------------------------------------------------------ */
+/* sliding-window attention with kept first positions, sigmoid weights */
+/* ------------------------------------------------------------------ */
+/* The step between a projection GEMM and semipd_window_attention, one launch.  Row t of qkv (row stride ld elements)
+ * holds q | k | v at columns 0, k_off, v_off.  q and k: + bias (bias_q [heads * qk_dim], bias_k, may be NULL), then the
+ * first rot_dims elements of every head as neighbouring pairs (2i, 2i + 1), pair i turned by positions[t] * inv_freq[i]
+ * (fp32); q in place, k to k_pool[loc[t]].  v: (v + bias_v) / sqrt(mean(.^2) + eps) per head to v_pool[loc[t]].  fp32
+ * arithmetic, pools [N, kv heads, size] of the activation type.  No reference counterpart. */
+int semipd_bias_rope_vnorm_kv_store(void* qkv, int64_t ld, int64_t num_tokens, int num_q_heads, int num_kv_heads,
+                                    int qk_dim, int v_dim, int64_t k_off, int64_t v_off, const void* bias_q,
+                                    const void* bias_k, const void* bias_v, const int64_t* positions,
+                                    const float* inv_freq, int rot_dims, float eps, void* k_pool, void* v_pool,
+                                    const int64_t* loc, int dtype, void* stream);
+/* Attention over the paged pools like semipd_local_attention (same description of the batch), with another mask and
+ * another kind of weight.  Mask: a query at position p sees key j <= p when p - j < window (window 0: every earlier key)
+ * or j < keep_first.  sigmoid == 1: key j weighs sigmoid(scale * q.k + head_bias[head]) (head_bias fp32 [heads], may be
+ * NULL) and the output is the plain sum of weight * value over the visible keys; sigmoid == 0: softmax over the visible
+ * keys, its denominator also holding exp(sink[head]) when sink is given.  The output is multiplied by out_scale.
+ * form as in semipd_local_attention.  No reference counterpart. */
+int semipd_window_attention(const void* q, int64_t q_ld, void* out, int64_t out_ld, const void* k_pool,
+                            const void* v_pool, const int32_t* req_to_token, int64_t req_to_token_stride,
+                            const int64_t* req_pool_indices, const int64_t* seq_lens, const int32_t* q_start,
+                            const int32_t* q_len, int64_t batch, int64_t num_tokens, int64_t max_q_len,
+                            int num_q_heads, int num_kv_heads, int qk_dim, int v_dim, float scale, int window,
+                            int keep_first, const float* head_bias, int sigmoid, const float* sink, float out_scale,
+                            int form, int dtype, void* stream);
+
+/* ------------------------------------------------------------------ */
+/* dynamic tanh, gated linear recurrence, routed squared ReLU          */
+/* ------------------------------------------------------------------ */
+/* tanh(alpha x) * weight + bias element by element (fp32; weight, bias [width] and the one-element alpha of `dtype`) on
+ * both sides of a residual stream: v = dyn_tanh_a(in) when `in` is given (rows fp32 if in_is_f32, else of `dtype`);
+ * with `residual` (fp32 rows): v += residual when accumulate is set or `in` is NULL, and residual <- v when `in` is given;
+ * out <- dyn_tanh_b(v) when weight_b is given, else out <- v.  Strides in elements.  No reference counterpart. */
+int semipd_dyn_tanh(const void* in, int64_t in_ld, int in_is_f32, const void* weight_a, const void* bias_a,
+                    const void* alpha_a, float* residual, int64_t residual_ld, int accumulate, const void* weight_b,
+                    const void* bias_b, const void* alpha_b, void* out, int64_t out_ld, int64_t rows, int64_t width,
+                    int dtype, void* stream);
+/* u [rows, experts * ff] in place: u[t, e * ff + f] <- w(t, e) * max(u, 0)^2 with w(t, e) = topk_weights[t, k] where
+ * topk_ids[t, k] == e, else 0.  No reference counterpart. */
+int semipd_routed_relu_square(void* u, int64_t ld, const float* topk_weights, const int32_t* topk_ids, int topk,
+                              int64_t rows, int64_t ff, int experts, int dtype, void* stream);
+/* minGRU over per-request state rows.  Row t of proj holds zlin | xlin | glin at columns z_off, x_off, g_off (`width`
+ * each).  Per channel: z = sigmoid(zlin + bias_z), u = xlin + bias_x, cand = u >= 0 ? u + 1/2 : sigmoid(u),
+ * S <- (1 - z) S + z cand, y = out_scale * S * silu(glin).  S is fp32 in state[state_indices[b]] (row stride state_ld):
+ * read unless request b's rows start its sequence (seq_lens[b] == number of its rows), written after its last row.
+ * Batch description (q_start / q_len / seq_lens / max_q_len) as in semipd_local_attention.  workspace (may be NULL;
+ * semipd_min_gru_workspace bytes) enables the chunked form for long portions.  No reference counterpart. */
+int semipd_min_gru(const void* proj, int64_t ld, int64_t z_off, int64_t x_off, int64_t g_off, const void* bias_z,
+                   const void* bias_x, void* y, int64_t y_ld, float* state, int64_t state_ld,
+                   const int64_t* state_indices, const int64_t* seq_lens, const int32_t* q_start, const int32_t* q_len,
+                   int64_t batch, int64_t num_tokens, int64_t max_q_len, int width, float out_scale, float* workspace,
+                   int64_t workspace_bytes, int dtype, void* stream);
+int64_t semipd_min_gru_workspace(int64_t num_tokens, int64_t batch, int width);
+
 #ifdef __cplusplus
 }
 #endif

@@ -5,6 +5,13 @@
 //    out in the activation type: the block "x <- x + norm(sublayer(x))" between two GEMMs in one launch, the residual
 //    never leaving fp32.  Input rows are of the activation type or fp32 (the final norm reads the stream itself).
 //  * bias_relu_square_kernel: u <- max(u + b, 0)^2 in place.
+//  * dyn_tanh_kernel: the element-wise squashing tanh(alpha x) * w + b that stands where a norm would (no row statistics),
+//    fp32.  One launch is the seam between two sublayers of a block with a squashing before AND after each sublayer:
+//    stream += dyn_tanh_a(sublayer output), then out = dyn_tanh_b(stream) for the next sublayer's GEMM; either half may
+//    be left out (the first squashing of a model, the last one in front of the vocabulary head).
+//  * routed_relu_square_kernel: experts evaluated side by side on every token (one GEMM over the stacked up-projections):
+//    u[t, e * F + f] <- w(t, e) * max(u, 0)^2 with w the routing weight of expert e for token t, 0 when e is not one of the
+//    token's experts, so that ONE GEMM over the stacked down-projections gives the weighted sum of the chosen experts.
 #include "common.h"
 
 namespace semipd {
@@ -176,6 +183,83 @@ __global__ void __launch_bounds__(256) bias_relu_square_kernel(T* __restrict__ u
   }
 }
 
+
+// ------------------------------------------------------------------------------------------------ dynamic tanh
+// V elements per thread (V = 8: 16-byte accesses on 16-bit rows; V = 1: any width and alignment)
+template <typename T, typename TIn, int V>
+__global__ void __launch_bounds__(256) dyn_tanh_kernel(const TIn* __restrict__ y, int64_t y_ld, const T* __restrict__ wa,
+                                                       const T* __restrict__ ba, const T* __restrict__ alpha_a,
+                                                       float* __restrict__ residual, int64_t res_ld, int accumulate,
+                                                       const T* __restrict__ wb, const T* __restrict__ bb,
+                                                       const T* __restrict__ alpha_b, T* __restrict__ out, int64_t out_ld,
+                                                       int64_t rows, int64_t width) {
+  const int64_t per_row = width / V, n = rows * per_row;
+  const float aa = alpha_a ? Elem<T>::to_f(alpha_a[0]) : 0.f, ab = alpha_b ? Elem<T>::to_f(alpha_b[0]) : 0.f;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / per_row, c = (i - r * per_row) * V;
+    float v[V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) v[k] = 0.f;
+    if (y) {
+      if constexpr (V == 8 && sizeof(TIn) == 2) {
+        const Vec16<TIn> a = load16(y + r * y_ld + c);
+#pragma unroll
+        for (int k = 0; k < V; ++k) v[k] = Elem<TIn>::to_f(a.e[k]);
+      } else {
+#pragma unroll
+        for (int k = 0; k < V; ++k) v[k] = Elem<TIn>::to_f(y[r * y_ld + c + k]);
+      }
+#pragma unroll
+      for (int k = 0; k < V; ++k) v[k] = tanhf(aa * v[k]) * Elem<T>::to_f(wa[c + k]) + Elem<T>::to_f(ba[c + k]);
+    }
+    if (residual) {
+      float* rp = residual + r * res_ld + c;
+      if (accumulate || !y) {
+#pragma unroll
+        for (int k = 0; k < V; ++k) v[k] += rp[k];
+      }
+      if (y) {
+#pragma unroll
+        for (int k = 0; k < V; ++k) rp[k] = v[k];
+      }
+    }
+    if (out) {
+      if (wb) {
+#pragma unroll
+        for (int k = 0; k < V; ++k) v[k] = tanhf(ab * v[k]) * Elem<T>::to_f(wb[c + k]) + Elem<T>::to_f(bb[c + k]);
+      }
+      T* op = out + r * out_ld + c;
+      if constexpr (V == 8 && sizeof(T) == 2) {
+        Vec16<T> o;
+#pragma unroll
+        for (int k = 0; k < V; ++k) o.e[k] = Elem<T>::from_f(v[k]);
+        store16(op, o);
+      } else {
+#pragma unroll
+        for (int k = 0; k < V; ++k) op[k] = Elem<T>::from_f(v[k]);
+      }
+    }
+  }
+}
+
+// one thread per element of u [rows, experts * ff]
+template <typename T>
+__global__ void __launch_bounds__(256) routed_relu_square_kernel(T* __restrict__ u, int64_t ld, const float* __restrict__ topk_weights,
+                                                                 const int32_t* __restrict__ topk_ids, int topk, int64_t rows,
+                                                                 int64_t ff, int experts) {
+  const int64_t width = ff * experts, n = rows * width;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / width, c = i - r * width;
+    const int e = (int)(c / ff);
+    float wgt = 0.f;
+    for (int k = 0; k < topk; ++k)
+      if (topk_ids[r * topk + k] == e) wgt = topk_weights[r * topk + k];
+    float v = Elem<T>::to_f(u[r * ld + c]);
+    v = v > 0.f ? v * v * wgt : 0.f;
+    u[r * ld + c] = Elem<T>::from_f(v);
+  }
+}
+
 }  // namespace semipd
 
 using namespace semipd;
@@ -244,4 +328,48 @@ extern "C" int semipd_bias_relu_square(void* u, int64_t ld, const void* bias, in
                         hipLaunchKernelGGL((bias_relu_square_kernel<T>), dim3(blocks), dim3(256), 0, as_stream(stream), (T*)u, ld,
                                            (const T*)bias, rows, width));
   return launch_status("bias_relu_square");
+}
+
+extern "C" int semipd_dyn_tanh(const void* in, int64_t in_ld, int in_is_f32, const void* weight_a, const void* bias_a,
+                               const void* alpha_a, float* residual, int64_t residual_ld, int accumulate, const void* weight_b,
+                               const void* bias_b, const void* alpha_b, void* out, int64_t out_ld, int64_t rows, int64_t width,
+                               int dtype, void* stream) {
+  SEMIPD_CHECK_ARG(rows >= 0 && width > 0, SEMIPD_EINVAL, "dyn_tanh: bad sizes");
+  if (rows == 0) return 0;
+  SEMIPD_CHECK_ARG((in || residual) && (residual || out), SEMIPD_EINVAL, "dyn_tanh: nothing to read or nothing to write");
+  SEMIPD_CHECK_ARG(!in || (weight_a && bias_a && alpha_a), SEMIPD_EINVAL, "dyn_tanh: the input's weight, bias and alpha come together");
+  SEMIPD_CHECK_ARG((weight_b == nullptr) == (bias_b == nullptr) && (weight_b == nullptr) == (alpha_b == nullptr), SEMIPD_EINVAL,
+                   "dyn_tanh: the output's weight, bias and alpha come together");
+  SEMIPD_CHECK_ARG(!weight_b || out, SEMIPD_EINVAL, "dyn_tanh: output parameters without an output");
+  const int64_t esz = dtype == SEMIPD_F32 ? 4 : 2, in_esz = in_is_f32 ? 4 : esz;
+  const bool vec = width % 8 == 0 && (!in || (aligned16(in) && (in_ld * in_esz) % 16 == 0)) &&
+                   (!residual || (aligned16(residual) && residual_ld % 4 == 0)) && (!out || (aligned16(out) && (out_ld * esz) % 16 == 0));
+  const int64_t n = rows * width / (vec ? 8 : 1);
+  const unsigned blocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
+#define SEMIPD_DYT(TIN, VV)                                                                                                     \
+  hipLaunchKernelGGL((dyn_tanh_kernel<T, TIN, VV>), dim3(blocks), dim3(256), 0, as_stream(stream), (const TIN*)in, in_ld,          \
+                     (const T*)weight_a, (const T*)bias_a, (const T*)alpha_a, residual, residual_ld, accumulate,                 \
+                     (const T*)weight_b, (const T*)bias_b, (const T*)alpha_b, (T*)out, out_ld, rows, width)
+  SEMIPD_DISPATCH_DTYPE(dtype, T, {
+    if (in_is_f32 && vec) SEMIPD_DYT(float, 8);
+    else if (in_is_f32) SEMIPD_DYT(float, 1);
+    else if (vec) SEMIPD_DYT(T, 8);
+    else SEMIPD_DYT(T, 1);
+  });
+#undef SEMIPD_DYT
+  return launch_status("dyn_tanh");
+}
+
+extern "C" int semipd_routed_relu_square(void* u, int64_t ld, const float* topk_weights, const int32_t* topk_ids, int topk,
+                                         int64_t rows, int64_t ff, int experts, int dtype, void* stream) {
+  SEMIPD_CHECK_ARG(rows >= 0 && ff > 0 && experts > 0 && topk > 0 && topk <= experts && ld >= ff * experts, SEMIPD_EINVAL,
+                   "routed_relu_square: bad sizes");
+  if (rows == 0) return 0;
+  SEMIPD_CHECK_ARG(u && topk_weights && topk_ids, SEMIPD_EINVAL, "routed_relu_square: null pointer");
+  const int64_t n = rows * ff * experts;
+  const unsigned blocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
+  SEMIPD_DISPATCH_DTYPE(dtype, T,
+                        hipLaunchKernelGGL((routed_relu_square_kernel<T>), dim3(blocks), dim3(256), 0, as_stream(stream), (T*)u,
+                                           ld, topk_weights, topk_ids, topk, rows, ff, experts));
+  return launch_status("routed_relu_square");
 }

@@ -13,6 +13,14 @@
 //    through transposing reads of a row-major LDS tile, the next step's loads in flight during the current one.
 //  * local_attention_decode_kernel (bf16 / f16): one workgroup per (request, kv head); the waves split the visible keys,
 //    the q heads of the group are the MFMA's columns, partials meet in LDS.
+//
+// The same walks serve a second family of masks and weights (semipd_window_attention):
+//  * mask: the last `window` positions up to the query, plus the first `keep_first` positions of the sequence, which stay
+//    visible at their true positions however far the window has moved on (window 0: the block mask above);
+//  * weights: with `sigmoid` set every visible key weighs sigmoid(score + head_bias[head]) on its own -- no maximum, no
+//    denominator, no sink -- and the result is the plain weighted sum of the value rows, times out_scale.
+//  * bias_rope_vnorm_kv_store_kernel, the step in front of it: projection biases, rotation of neighbouring pairs of q and k
+//    by angles position * inv_freq[pair] (fp32 product, sincosf), values scaled to unit RMS; k and v into the pools.
 #include "common.h"
 #include "mfma_frag.h"
 
@@ -109,6 +117,73 @@ __global__ void __launch_bounds__(256) unit_norm_kv_store_vec_kernel(
   }
 }
 
+
+// ------------------------------------------------------------------------------------------------ bias + rotation + value norm + store
+// One wave per (token, head) of q | k | v.  q and k: x + bias, then the first `rot` elements of the head as rot / 2 neighbouring
+// pairs (2i, 2i + 1), pair i turned by the angle pos * inv_freq[i] (fp32 product; sincosf reduces the argument itself); the
+// rest of the head passes.  q in place, k into the key pool.  v: (x + bias) / sqrt(mean((x + bias)^2) + eps) into the value
+// pool.  Everything in fp32, one rounding on the way out.
+template <typename T>
+__global__ void __launch_bounds__(256) bias_rope_vnorm_kv_store_kernel(
+    T* __restrict__ qkv, int64_t ld, int64_t num_tokens, int H, int G, int D, int E, int64_t k_off, int64_t v_off,
+    const T* __restrict__ bq, const T* __restrict__ bk, const T* __restrict__ bv, const int64_t* __restrict__ positions,
+    const float* __restrict__ inv_freq, int rot, float eps, T* __restrict__ k_pool, T* __restrict__ v_pool,
+    const int64_t* __restrict__ loc) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int items = H + 2 * G;
+  const int64_t item = (int64_t)blockIdx.x * 4 + wave;
+  if (item >= num_tokens * items) return;
+  const int64_t t = item / items;
+  const int h = (int)(item % items);
+  T* row = qkv + t * ld;
+  if (h < H + G) {
+    const bool is_q = h < H;
+    const int hh = is_q ? h : h - H;
+    T* src = is_q ? row + (int64_t)hh * D : row + k_off + (int64_t)hh * D;
+    const T* bias = is_q ? bq : bk;
+    T* dst = is_q ? src : k_pool + (loc[t] * G + hh) * D;
+    const float pos = (float)positions[t];
+    for (int i = lane; i < rot / 2; i += 64) {
+      float x0 = Elem<T>::to_f(src[2 * i]), x1 = Elem<T>::to_f(src[2 * i + 1]);
+      if (bias) {
+        x0 += Elem<T>::to_f(bias[hh * D + 2 * i]);
+        x1 += Elem<T>::to_f(bias[hh * D + 2 * i + 1]);
+      }
+      float sn, cs;
+      sincosf(pos * inv_freq[i], &sn, &cs);
+      dst[2 * i] = Elem<T>::from_f(x0 * cs - x1 * sn);
+      dst[2 * i + 1] = Elem<T>::from_f(x1 * cs + x0 * sn);
+    }
+    for (int d = rot + lane; d < D; d += 64) {
+      float x = Elem<T>::to_f(src[d]);
+      if (bias) x += Elem<T>::to_f(bias[hh * D + d]);
+      dst[d] = Elem<T>::from_f(x);
+    }
+  } else {
+    const int g = h - H - G;
+    const T* src = row + v_off + (int64_t)g * E;
+    T* dst = v_pool + (loc[t] * G + g) * E;
+    float x[4], ss = 0.f;      // E <= 256
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int e = lane + 64 * u;
+      x[u] = 0.f;
+      if (e < E) {
+        x[u] = Elem<T>::to_f(src[e]);
+        if (bv) x[u] += Elem<T>::to_f(bv[g * E + e]);
+        ss += x[u] * x[u];
+      }
+    }
+    ss = wave_sum(ss);
+    const float r = 1.0f / sqrtf(ss / (float)E + eps);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int e = lane + 64 * u;
+      if (e < E) dst[e] = Elem<T>::from_f(x[u] * r);
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ shared pieces
 struct LocalAttnArgs {
   const void* q; int64_t q_ld;
@@ -124,7 +199,22 @@ struct LocalAttnArgs {
   float scale, cap;
   int chunk;
   int64_t n_tiles;       // prompt form: 64-row tiles, an upper bound (tiles past the last request's do nothing)
+  int window, keep_first;          // window > 0: keys pos - window + 1 .. pos and keys 0 .. keep_first - 1
+  const float* head_bias;          // sigmoid weights: added to the score of every key of the head (may be NULL)
+  int sigmoid;                     // 0: softmax over the visible keys (+ sink); 1: independent sigmoid weights
+  float out_scale;
 };
+
+// first visible position of the contiguous range that ends at the query (the kept first positions come on top)
+__device__ __forceinline__ int64_t range_lo(const LocalAttnArgs& a, int64_t pos) {
+  if (a.window > 0) return pos - a.window + 1 > 0 ? pos - a.window + 1 : 0;
+  return a.chunk > 0 ? (pos / a.chunk) * a.chunk : 0;
+}
+// how many of the kept first positions lie in front of that range
+__device__ __forceinline__ int64_t kept_before(const LocalAttnArgs& a, int64_t lo) {
+  if (a.window <= 0) return 0;
+  return a.keep_first < lo ? a.keep_first : lo;
+}
 
 __device__ __forceinline__ float capped(float s, float scale, float cap) {
   s *= scale;
@@ -166,51 +256,62 @@ __global__ void __launch_bounds__(256) local_attention_rows_kernel(LocalAttnArgs
   for (int d = lane; d < D; d += 64) q_lds[wave][d] = Elem<T>::to_f(q[d]);
   __builtin_amdgcn_wave_barrier();
   const int32_t* row = a.req_to_token + a.req_pool_indices[b] * a.r2t_stride;
-  const int64_t lo = a.chunk > 0 ? (pos / a.chunk) * a.chunk : 0;
+  const int64_t lo = range_lo(a, pos), n_first = kept_before(a, lo);
   const T* kp = (const T*)a.k_pool;
   const T* vp = (const T*)a.v_pool;
-  float m = -INFINITY, l = 0.f, acc[4] = {0.f, 0.f, 0.f, 0.f};
+  const bool sig = a.sigmoid != 0;
+  const float hb = (sig && a.head_bias) ? a.head_bias[h] : 0.f;
+  float m = sig ? 0.f : -INFINITY, l = 0.f, acc[4] = {0.f, 0.f, 0.f, 0.f};
   constexpr int V = Elem<T>::kVec;
-  for (int64_t j0 = lo; j0 <= pos; j0 += 64) {
-    const int64_t j = j0 + lane;
-    const bool valid = j <= pos;
-    const int slot = valid ? row[j] : 0;
-    float s = -INFINITY;
-    if (valid) {
-      const T* k = kp + ((int64_t)slot * G + g) * D;
-      float dot = 0.f;
-      if ((D % V) == 0) {
-        for (int d = 0; d < D; d += V) {
-          const Vec16<T> kv = load16(k + d);
+  // the kept first positions (none without a window), then the range that ends at the query
+  for (int seg = n_first > 0 ? 0 : 1; seg < 2; ++seg) {
+    const int64_t j_begin = seg == 0 ? 0 : lo, j_last = seg == 0 ? n_first - 1 : pos;
+    for (int64_t j0 = j_begin; j0 <= j_last; j0 += 64) {
+      const int64_t j = j0 + lane;
+      const bool valid = j <= j_last;
+      const int slot = valid ? row[j] : 0;
+      float s = -INFINITY;
+      if (valid) {
+        const T* k = kp + ((int64_t)slot * G + g) * D;
+        float dot = 0.f;
+        if ((D % V) == 0) {
+          for (int d = 0; d < D; d += V) {
+            const Vec16<T> kv = load16(k + d);
 #pragma unroll
-          for (int u = 0; u < V; ++u) dot += q_lds[wave][d + u] * Elem<T>::to_f(kv.e[u]);
+            for (int u = 0; u < V; ++u) dot += q_lds[wave][d + u] * Elem<T>::to_f(kv.e[u]);
+          }
+        } else {
+          for (int d = 0; d < D; ++d) dot += q_lds[wave][d] * Elem<T>::to_f(k[d]);
         }
-      } else {
-        for (int d = 0; d < D; ++d) dot += q_lds[wave][d] * Elem<T>::to_f(k[d]);
+        s = capped(dot, a.scale, a.cap);
       }
-      s = capped(dot, a.scale, a.cap);
-    }
-    const float m_new = fmaxf(m, wave_max(s));
-    const float alpha = expf(m - m_new);      // first tile: exp(-inf) = 0
-    const float p = valid ? expf(s - m_new) : 0.f;
-    l = l * alpha + wave_sum(p);
+      float p;
+      if (sig) {
+        p = valid ? 1.0f / (1.0f + expf(-(s + hb))) : 0.f;
+      } else {
+        const float m_new = fmaxf(m, wave_max(s));
+        const float alpha = expf(m - m_new);      // first tile: exp(-inf) = 0
+        p = valid ? expf(s - m_new) : 0.f;
+        l = l * alpha + wave_sum(p);
 #pragma unroll
-    for (int u = 0; u < 4; ++u) acc[u] *= alpha;
-    m = m_new;
-    const int n = (int)((pos - j0 + 1) < 64 ? (pos - j0 + 1) : 64);
-    for (int jj = 0; jj < n; ++jj) {
-      const float pj = __shfl(p, jj, 64);
-      const int sj = __shfl(slot, jj, 64);
-      const T* v = vp + ((int64_t)sj * G + g) * E;
+        for (int u = 0; u < 4; ++u) acc[u] *= alpha;
+        m = m_new;
+      }
+      const int n = (int)((j_last - j0 + 1) < 64 ? (j_last - j0 + 1) : 64);
+      for (int jj = 0; jj < n; ++jj) {
+        const float pj = __shfl(p, jj, 64);
+        const int sj = __shfl(slot, jj, 64);
+        const T* v = vp + ((int64_t)sj * G + g) * E;
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int e = lane + 64 * u;
-        if (e < E) acc[u] += pj * Elem<T>::to_f(v[e]);
+        for (int u = 0; u < 4; ++u) {
+          const int e = lane + 64 * u;
+          if (e < E) acc[u] += pj * Elem<T>::to_f(v[e]);
+        }
       }
     }
   }
-  if (a.sink != nullptr) l += expf(a.sink[h] - m);
-  const float inv = 1.0f / l;
+  if (!sig && a.sink != nullptr) l += expf(a.sink[h] - m);
+  const float inv = sig ? a.out_scale : a.out_scale / l;
   T* o = (T*)a.out + t * a.out_ld + (int64_t)h * E;
   const T* gt = a.gate ? (const T*)a.gate + t * a.gate_ld + (int64_t)h * E : nullptr;
 #pragma unroll
@@ -714,6 +815,8 @@ extern "C" int semipd_unit_norm_kv_store(void* qkv, int64_t ld, int64_t num_toke
   return launch_status("unit_norm_kv_store");
 }
 
+static int launch_local_attention(LocalAttnArgs a, int64_t max_q_len, int form, int dtype, void* stream);
+
 extern "C" int semipd_local_attention(const void* q, int64_t q_ld, const void* gate, int64_t gate_ld, void* out, int64_t out_ld,
                                       const void* k_pool, const void* v_pool, const int32_t* req_to_token,
                                       int64_t req_to_token_stride, const int64_t* req_pool_indices, const int64_t* seq_lens,
@@ -721,22 +824,47 @@ extern "C" int semipd_local_attention(const void* q, int64_t q_ld, const void* g
                                       int64_t max_q_len, int num_q_heads, int num_kv_heads, int qk_dim, int v_dim,
                                       const float* sink, float scale, float logit_cap, int chunk, int form, int dtype,
                                       void* stream) {
+  SEMIPD_CHECK_ARG(chunk >= 0, SEMIPD_EINVAL, "local_attention: bad chunk");
+  LocalAttnArgs a{q, q_ld, gate, gate_ld, out, out_ld, k_pool, v_pool, req_to_token, req_to_token_stride, req_pool_indices,
+                  seq_lens, q_start, q_len, batch, num_tokens, num_q_heads, num_kv_heads, qk_dim, v_dim, sink, scale, logit_cap,
+                  chunk, 0, 0, 0, nullptr, 0, 1.0f};
+  return launch_local_attention(a, max_q_len, form, dtype, stream);
+}
+
+extern "C" int semipd_window_attention(const void* q, int64_t q_ld, void* out, int64_t out_ld, const void* k_pool,
+                                       const void* v_pool, const int32_t* req_to_token, int64_t req_to_token_stride,
+                                       const int64_t* req_pool_indices, const int64_t* seq_lens, const int32_t* q_start,
+                                       const int32_t* q_len, int64_t batch, int64_t num_tokens, int64_t max_q_len,
+                                       int num_q_heads, int num_kv_heads, int qk_dim, int v_dim, float scale, int window,
+                                       int keep_first, const float* head_bias, int sigmoid, const float* sink, float out_scale,
+                                       int form, int dtype, void* stream) {
+  SEMIPD_CHECK_ARG(window >= 0 && keep_first >= 0, SEMIPD_EINVAL, "window_attention: bad window or number of kept positions");
+  SEMIPD_CHECK_ARG(window > 0 || keep_first == 0, SEMIPD_EINVAL, "window_attention: kept first positions need a window");
+  SEMIPD_CHECK_ARG(!sigmoid || sink == nullptr, SEMIPD_EINVAL, "window_attention: sigmoid weights have no denominator for a sink");
+  LocalAttnArgs a{q, q_ld, nullptr, 0, out, out_ld, k_pool, v_pool, req_to_token, req_to_token_stride, req_pool_indices,
+                  seq_lens, q_start, q_len, batch, num_tokens, num_q_heads, num_kv_heads, qk_dim, v_dim, sink, scale, 0.f,
+                  0, 0, window, keep_first, head_bias, sigmoid ? 1 : 0, out_scale};
+  return launch_local_attention(a, max_q_len, form, dtype, stream);
+}
+
+static int launch_local_attention(LocalAttnArgs a, int64_t max_q_len, int form, int dtype, void* stream) {
+  const void* q = a.q; const void* gate = a.gate; void* out = a.out; const void* k_pool = a.k_pool; const void* v_pool = a.v_pool;
+  const int64_t q_ld = a.q_ld, gate_ld = a.gate_ld, out_ld = a.out_ld, batch = a.batch, num_tokens = a.num_tokens;
+  const int32_t* q_start = a.q_start; const int32_t* q_len = a.q_len;
+  const int num_q_heads = a.H, num_kv_heads = a.G, qk_dim = a.D, v_dim = a.E;
   SEMIPD_CHECK_ARG(batch >= 0 && num_tokens >= 0, SEMIPD_EINVAL, "local_attention: bad sizes");
   if (batch == 0 || num_tokens == 0) return 0;
   SEMIPD_CHECK_ARG(num_q_heads > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0, SEMIPD_ESHAPE,
                    "local_attention: %d query heads over %d key/value heads", num_q_heads, num_kv_heads);
   SEMIPD_CHECK_ARG(qk_dim > 0 && qk_dim <= 512 && v_dim > 0 && v_dim <= 256, SEMIPD_ESHAPE,
                    "local_attention: head sizes %d / %d (at most 512 / 256)", qk_dim, v_dim);
-  SEMIPD_CHECK_ARG(q && out && k_pool && v_pool && req_to_token && req_pool_indices && seq_lens, SEMIPD_EINVAL,
+  SEMIPD_CHECK_ARG(q && out && k_pool && v_pool && a.req_to_token && a.req_pool_indices && a.seq_lens, SEMIPD_EINVAL,
                    "local_attention: null pointer");
   SEMIPD_CHECK_ARG((q_start == nullptr) == (q_len == nullptr), SEMIPD_EINVAL, "local_attention: q_start and q_len come together");
   SEMIPD_CHECK_ARG(q_start != nullptr || num_tokens == batch, SEMIPD_EINVAL, "local_attention: one row per request without q_start");
-  SEMIPD_CHECK_ARG(chunk >= 0 && logit_cap >= 0.f, SEMIPD_EINVAL, "local_attention: bad chunk or cap");
-  LocalAttnArgs a{q, q_ld, gate, gate_ld, out, out_ld, k_pool, v_pool, req_to_token, req_to_token_stride, req_pool_indices,
-                  seq_lens, q_start, q_len, batch, num_tokens, num_q_heads, num_kv_heads, qk_dim, v_dim, sink, scale, logit_cap,
-                  chunk, 0};
+  SEMIPD_CHECK_ARG(a.cap >= 0.f, SEMIPD_EINVAL, "local_attention: bad cap");
   const bool half = dtype == SEMIPD_BF16 || dtype == SEMIPD_F16;
-  const bool mfma_ok = half && local_mfma_shape_ok(qk_dim, v_dim) && aligned16(q) && q_ld % 8 == 0 && aligned16(k_pool) &&
+  const bool mfma_ok = half && a.window == 0 && !a.sigmoid && a.out_scale == 1.0f && local_mfma_shape_ok(qk_dim, v_dim) && aligned16(q) && q_ld % 8 == 0 && aligned16(k_pool) &&
                        aligned16(v_pool) && aligned16(out) && out_ld % 8 == 0 &&
                        (gate == nullptr || (aligned16(gate) && gate_ld % 8 == 0));
   SEMIPD_CHECK_ARG(form != 2 || mfma_ok, SEMIPD_ESHAPE, "local_attention: the matrix-core forms do not take this shape or type");
@@ -792,4 +920,29 @@ extern "C" int semipd_local_attention(const void* q, int64_t q_ld, const void* g
 extern "C" int semipd_local_attention_mfma_supported(int num_q_heads, int num_kv_heads, int qk_dim, int v_dim, int dtype) {
   return (dtype == SEMIPD_BF16 || dtype == SEMIPD_F16) && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0 &&
          local_mfma_shape_ok(qk_dim, v_dim);
+}
+
+extern "C" int semipd_bias_rope_vnorm_kv_store(void* qkv, int64_t ld, int64_t num_tokens, int num_q_heads, int num_kv_heads,
+                                               int qk_dim, int v_dim, int64_t k_off, int64_t v_off, const void* bias_q,
+                                               const void* bias_k, const void* bias_v, const int64_t* positions,
+                                               const float* inv_freq, int rot_dims, float eps, void* k_pool, void* v_pool,
+                                               const int64_t* loc, int dtype, void* stream) {
+  SEMIPD_CHECK_ARG(num_tokens >= 0 && num_q_heads > 0 && num_kv_heads > 0 && qk_dim > 0 && v_dim > 0 && v_dim <= 256, SEMIPD_EINVAL,
+                   "bias_rope_vnorm_kv_store: bad sizes (value rows of at most 256 elements)");
+  SEMIPD_CHECK_ARG(rot_dims >= 0 && rot_dims <= qk_dim && rot_dims % 2 == 0, SEMIPD_EINVAL,
+                   "bias_rope_vnorm_kv_store: %d rotated elements of a head of %d", rot_dims, qk_dim);
+  if (num_tokens == 0) return 0;
+  SEMIPD_CHECK_ARG(qkv && k_pool && v_pool && loc && positions && (rot_dims == 0 || inv_freq), SEMIPD_EINVAL,
+                   "bias_rope_vnorm_kv_store: null pointer");
+  SEMIPD_CHECK_ARG(ld >= v_off + (int64_t)num_kv_heads * v_dim && k_off >= (int64_t)num_q_heads * qk_dim &&
+                       v_off >= k_off + (int64_t)num_kv_heads * qk_dim,
+                   SEMIPD_EINVAL, "bias_rope_vnorm_kv_store: column ranges overlap or leave the row");
+  const int64_t items = num_tokens * (num_q_heads + 2 * num_kv_heads);
+  const unsigned blocks = (unsigned)((items + 3) / 4);
+  SEMIPD_DISPATCH_DTYPE(dtype, T,
+                        hipLaunchKernelGGL((bias_rope_vnorm_kv_store_kernel<T>), dim3(blocks), dim3(256), 0, as_stream(stream),
+                                           (T*)qkv, ld, num_tokens, num_q_heads, num_kv_heads, qk_dim, v_dim, k_off, v_off,
+                                           (const T*)bias_q, (const T*)bias_k, (const T*)bias_v, positions, inv_freq, rot_dims,
+                                           eps, (T*)k_pool, (T*)v_pool, loc));
+  return launch_status("bias_rope_vnorm_kv_store");
 }

@@ -153,9 +153,19 @@ _SIGNATURES = {
     "semipd_local_attention": [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32,
                                _i32, _i32, _vp, _f32, _f32, _i32, _i32, _i32, _vp],
     "semipd_local_attention_mfma_supported": [_i32, _i32, _i32, _i32, _i32],
+    "semipd_bias_rope_vnorm_kv_store": [_vp, _i64, _i64, _i32, _i32, _i32, _i32, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _i32, _f32,
+                                        _vp, _vp, _vp, _i32, _vp],
+    "semipd_window_attention": [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32, _i32,
+                                _i32, _f32, _i32, _i32, _vp, _i32, _vp, _f32, _i32, _i32, _vp],
+    "semipd_dyn_tanh": [_vp, _i64, _i32, _vp, _vp, _vp, _vp, _i64, _i32, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp],
+    "semipd_routed_relu_square": [_vp, _i64, _vp, _vp, _i32, _i64, _i64, _i32, _i32, _vp],
+    "semipd_min_gru": [_vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32,
+                       _f32, _vp, _i64, _i32, _vp],
+    "semipd_min_gru_workspace": [_i64, _i64, _i32],
 }
 _RESTYPES = {"semipd_last_error": C.c_char_p, "semipd_lm_head_argmax_workspace": _sz,
-             "semipd_linear_workspace": _sz, "semipd_stream_linear_workspace": _sz, "semipd_dense_gemm_report": _sz, "semipd_ar_meta_size": _sz, "semipd_ar_region_size": _sz}
+             "semipd_linear_workspace": _sz, "semipd_stream_linear_workspace": _sz, "semipd_dense_gemm_report": _sz, "semipd_ar_meta_size": _sz, "semipd_ar_region_size": _sz,
+             "semipd_min_gru_workspace": _i64}
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 
@@ -168,6 +178,7 @@ CORE_SOURCES = ("elementwise.hip", "skinny_gemm.hip", "stream_linear.hip", "gemm
                 "moe_tiled_gemm.hip", "sampling.hip", "ipc.hip")          # pools, GEMMs, logits, sampler, streams
 MODEL_SOURCES = {
     "Kudirax": ("local_attention.hip", "layernorm.hip"),
+    "Tigotar": ("local_attention.hip", "layernorm.hip", "recurrent.hip"),
 }
 
 

@@ -272,6 +272,33 @@ class HipAttnBackend(AttentionBackend):
             kt.stop("decode_attention" if forward_batch.forward_mode.is_decode() else "extend_attention", t0, 0.0, 0.0)
         return o
 
+    # ---- sliding window with kept first positions, softmax or independent sigmoid weights --------------------------
+    def forward_window(self, q, layer, forward_batch: ForwardBatch, out=None, head_bias=None, sink=None, out_scale: float = 1.0):
+        """Like forward_local (keys and values already in the pool, one call for prompt portions, single tokens and decode
+        batches) for layers whose descriptor carries `window` / `keep_first` / `sigmoid_weights`: a query sees the last
+        `window` positions and the first `keep_first` of its sequence; with sigmoid weights every visible key weighs
+        sigmoid(score + head_bias[head]) without normalisation.  `out` may be a column range of a wider buffer (the input
+        of an output projection that other mixers write next to); the result is multiplied by out_scale."""
+        T = q.shape[0]
+        if out is None:
+            out = torch.empty((T, layer.tp_q_head_num * layer.v_head_dim), dtype=q.dtype, device=q.device)
+        pool = forward_batch.token_to_kv_pool
+        if forward_batch.forward_mode.is_decode():
+            q_start = q_len = None
+            max_q = 1
+        else:
+            q_start, q_len = forward_batch.extend_start_loc, forward_batch.extend_seq_lens
+            max_q = max(forward_batch.extend_seq_lens_cpu)
+        kt = self._timing()
+        t0 = kt.start() if kt else None
+        ops.window_attention_fwd(q, out, pool.get_key_buffer(layer.layer_id), pool.get_value_buffer(layer.layer_id),
+                                 self.req_to_token, forward_batch.req_pool_indices, forward_batch.seq_lens, q_start, q_len, max_q,
+                                 layer.scaling, layer.window, layer.keep_first, head_bias, layer.sigmoid_weights, sink,
+                                 out_scale, form=int(os.environ.get("SEMIPD_LOCAL_ATTN_FORM", "0")))
+        if kt:
+            kt.stop("decode_attention" if forward_batch.forward_mode.is_decode() else "extend_attention", t0, 0.0, 0.0)
+        return out
+
     # ---- decode: RoPE + KV store + attention + split merge in one launch -------------------------
     def fused_decode_waves(self, bs: int, head_dim: int, num_kv_splits: int = 0) -> int:
         """How a decode batch of `bs` requests goes from the qkv GEMM's planes to o_proj's input: 0 = the separate
@@ -337,7 +364,8 @@ class RadixAttention:
     layer id; forward() reshapes nothing and dispatches to the batch's backend."""
 
     def __init__(self, num_heads: int, head_dim: int, scaling: float, num_kv_heads: int, layer_id: int,
-                 logit_cap: float = 0.0, v_head_dim: int = -1, chunk_size: int = 0):
+                 logit_cap: float = 0.0, v_head_dim: int = -1, chunk_size: int = 0, window: int = 0, keep_first: int = 0,
+                 sigmoid_weights: bool = False):
         self.tp_q_head_num = num_heads
         self.tp_k_head_num = num_kv_heads
         self.tp_v_head_num = num_kv_heads
@@ -350,6 +378,9 @@ class RadixAttention:
         # block-local attention (HipAttnBackend.forward_local): a query sees the keys of its own block of chunk_size positions,
         # counted from the start of the sequence (0: all earlier keys)
         self.chunk_size = int(chunk_size)
+        # sliding window (HipAttnBackend.forward_window): the last `window` positions up to the query (0: all) plus the first
+        # `keep_first` positions of the sequence; sigmoid_weights: independent sigmoid weights instead of a softmax
+        self.window, self.keep_first, self.sigmoid_weights = int(window), int(keep_first), bool(sigmoid_weights)
 
     def forward(self, q, k, v, forward_batch: ForwardBatch, save_kv_cache: bool = True):
         return forward_batch.attn_backend.forward(q, k, v, self, forward_batch, save_kv_cache)

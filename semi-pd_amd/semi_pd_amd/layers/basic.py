@@ -70,6 +70,42 @@ class LayerNorm(nn.Module):
         return ops.layernorm(y, self.weight, self.bias, self.eps, residual=residual, in_bias=in_bias)
 
 
+class DynTanh(nn.Module):
+    """Dynamic tanh, the element-wise squashing tanh(alpha x) * weight + bias that stands where a norm would: no mean, no
+    variance, nothing that couples the elements of a row (csrc/layernorm.hip: semipd_dyn_tanh; fp32 arithmetic whatever the
+    activation type).  `forward` squashes rows (fp32 stream or activations); `seam` is the joint between two sublayers of
+    a block that squashes before and after each of them: stream += self(y), and what the next sublayer reads,
+    next_norm(stream), comes back in the activation type from the same launch."""
+
+    def __init__(self, hidden_size: int, dtype=None):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(hidden_size, dtype=dtype), requires_grad=False)
+        self.bias = nn.Parameter(torch.zeros(hidden_size, dtype=dtype), requires_grad=False)
+        self.alpha = nn.Parameter(torch.ones((), dtype=dtype), requires_grad=False)
+
+    @property
+    def params(self):
+        return (self.weight, self.bias, self.alpha)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """x [rows, width], of the activation type or fp32 -> squashed rows in the activation type."""
+        return ops.dyn_tanh(x, self.params)
+
+    def forward_stream(self, x: torch.Tensor, residual: torch.Tensor) -> None:
+        """residual (fp32, preallocated) <- self(x): the start of a residual stream."""
+        ops.dyn_tanh(x, self.params, residual=residual, accumulate=False, want_out=False)
+
+    def read_stream(self, residual: torch.Tensor) -> torch.Tensor:
+        """self(residual) in the activation type; the stream is left as it is."""
+        return ops.dyn_tanh(None, None, residual=residual, params_out=self.params)
+
+    def seam(self, y: torch.Tensor, residual: torch.Tensor, next_norm: Optional["DynTanh"] = None,
+             want_out: bool = True) -> Optional[torch.Tensor]:
+        """residual += self(y); returns next_norm(residual) (or the sum itself without next_norm) in the activation type."""
+        return ops.dyn_tanh(y, self.params, residual=residual, params_out=next_norm.params if next_norm is not None else None,
+                            want_out=want_out)
+
+
 class SiluAndMul(nn.Module):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return ops.silu_and_mul(x)
@@ -623,10 +659,11 @@ class LogitsProcessor(nn.Module):
     greedy batch the argmax is produced by the same HIP call (ops.lm_head_argmax); with TP>1 the
     local shard of the logits is computed, gathered and then reduced with ops.greedy_argmax."""
 
-    def __init__(self, vocab_size: int, final_logit_softcapping: Optional[float] = None):
+    def __init__(self, vocab_size: int, final_logit_softcapping: Optional[float] = None, logit_scale: float = 1.0):
         super().__init__()
         self.vocab_size = vocab_size
         self.final_logit_softcapping = final_logit_softcapping
+        self.logit_scale = float(logit_scale)     # the fp32 logits are multiplied by it (1: as they are)
 
     def forward(self, input_ids, hidden_states: torch.Tensor, lm_head: VocabParallelEmbedding,
                 forward_batch) -> LogitsProcessorOutput:
@@ -647,6 +684,9 @@ class LogitsProcessor(nn.Module):
             # rows >= vocab_size are padding (vocab_parallel_embedding.py pads to a multiple of 64)
             logits, ids = ops.lm_head_argmax(pruned.contiguous(), lm_head.weight[: self.vocab_size],
                                              return_logits=True)
+            if self.logit_scale != 1.0:
+                # (a positive factor keeps the argmax; anything else leaves it to the sampler)
+                return LogitsProcessorOutput(logits * self.logit_scale, next_token_ids=ids if self.logit_scale > 0 else None)
             return LogitsProcessorOutput(logits, next_token_ids=ids)
         if (_STREAM_LINEAR["enabled"] and pruned.dim() == 2 and pruned.shape[0] > LM_HEAD_FUSED_MAX_ROWS
                 and ops.gemm_tall_is_supported(pruned, lm_head.weight)):
@@ -664,6 +704,8 @@ class LogitsProcessor(nn.Module):
             logits = torch.matmul(pruned, lm_head.weight.T)
         logits = tensor_model_parallel_all_gather(logits)
         logits = logits[:, : self.vocab_size].float()
+        if self.logit_scale != 1.0:
+            logits = logits * self.logit_scale
         if self.final_logit_softcapping:
             logits = self.final_logit_softcapping * torch.tanh(logits / self.final_logit_softcapping)
         return LogitsProcessorOutput(logits)

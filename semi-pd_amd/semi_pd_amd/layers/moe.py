@@ -352,3 +352,110 @@ class FusedMoE(nn.Module):
         if self.reduce_results and get_tensor_model_parallel_world_size() > 1:
             out = tensor_model_parallel_all_reduce(out)
         return out
+
+
+# ---- experts without a gate branch: down(act(up(x))) ---------------------------------------------------------------------
+def _relu_square_(u: torch.Tensor) -> torch.Tensor:
+    return ops.bias_relu_square_(u, None)
+
+
+UNGATED_ACTIVATIONS = {"relu2": _relu_square_}
+
+
+def fused_experts_ungated(hidden_states: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, topk_weights: torch.Tensor,
+                          topk_ids: torch.Tensor, activation: str = "relu2") -> torch.Tensor:
+    """Experts that are a plain two-layer feed-forward, down(act(up(x))), on the grouped GEMMs of fused_experts (bf16 / f16):
+    align -> GEMM(up) -> activation -> GEMM(down) x routing weight -> sum over the token's experts.  hidden [T, K];
+    w_up [E, F, K]; w_down [E, K, F]; returns [T, K].  Decode-sized calls take the grouped weight-streaming kernel where
+    its shapes allow, prefill-sized ones the tiled kernel, everything else the general grouped kernel."""
+    act = UNGATED_ACTIVATIONS[activation]
+    T, K = hidden_states.shape
+    E, F, _ = w_up.shape
+    if T == 0:
+        return hidden_states.new_zeros((0, K))
+    topk = topk_ids.shape[1]
+    dev, dt = hidden_states.device, hidden_states.dtype
+    numel = T * topk
+    tall = (numel >= MOE_TALL_MIN_ROWS and numel >= MOE_TALL_MIN_ROWS_PER_EXPERT * E
+            and ops.moe_gemm_tall_is_supported(hidden_states, w_up, False) and F % 64 == 0 and K % 16 == 0)
+    small = (MOE_STREAM_DECODE and T <= MOE_STREAM_MAX_TOKENS and ops.moe_stream_gemm_is_supported(hidden_states, w_up, False)
+             and F % 128 == 0 and K % 16 == 0)
+    tall_block = ops.MOE_TALL_BLOCK_M
+    if not tall and not small and (numel >= MOE_MID_MIN_ROWS_PER_EXPERT * E and ops.moe_gemm_tall_is_supported(hidden_states, w_up, False)
+                                   and F % 64 == 0 and K % 16 == 0):
+        tall, tall_block = True, 128
+    block_m = tall_block if tall else (min(64, 16 * -(-T // 16)) if small else MOE_BLOCK_M)
+    max_sorted = -(-(numel + E * (block_m - 1)) // block_m) * block_m
+    sorted_ids = torch.empty(max_sorted, dtype=torch.int32, device=dev)
+    expert_ids = torch.empty((max_sorted + block_m - 1) // block_m, dtype=torch.int32, device=dev)
+    num_post_pad = torch.empty(1, dtype=torch.int32, device=dev)
+    cumsum = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    ops.moe_align_block_size(topk_ids, E, block_m, sorted_ids, expert_ids, num_post_pad, None, cumsum)
+    c1 = torch.empty((numel, F), dtype=dt, device=dev)
+    c3 = torch.empty((numel, K), dtype=dt, device=dev)
+    wts = topk_weights.reshape(-1)
+    if small:
+        ops.moe_stream_gemm(hidden_states, w_up, c1, None, sorted_ids, expert_ids, num_post_pad, numel, topk, False, block_m)
+        act(c1)
+        ops.moe_stream_gemm(c1, w_down, c3, wts, sorted_ids, expert_ids, num_post_pad, numel, 1, True, block_m)
+    elif tall:
+        ops.moe_gemm_tall(hidden_states, w_up, c1, None, sorted_ids, expert_ids, num_post_pad, numel, topk, False, False,
+                          block_m=block_m)
+        act(c1)
+        ops.moe_gemm_tall(c1, w_down, c3, wts, sorted_ids, expert_ids, num_post_pad, numel, 1, True, False, block_m=block_m)
+    else:
+        ops.moe_grouped_gemm(hidden_states, w_up, c1, None, sorted_ids, expert_ids, num_post_pad, numel, topk, False, block_m)
+        act(c1)
+        ops.moe_grouped_gemm(c1, w_down, c3, wts, sorted_ids, expert_ids, num_post_pad, numel, 1, True, block_m)
+    return ops.moe_sum(c3.view(T, topk, K))
+
+
+def side_by_side_experts(hidden_states: torch.Tensor, w_up: torch.Tensor, w_down_cat: torch.Tensor, topk_weights: torch.Tensor,
+                         topk_ids: torch.Tensor) -> torch.Tensor:
+    """The same mixture with every expert evaluated on every token through two plain GEMMs: up-projections stacked
+    ([E * F, K], a view of w_up), squared ReLU times the routing weight of the column's expert (0 for experts the token does
+    not use), down-projections side by side along the input axis (w_down_cat [K, E * F]).  E / top-k times the arithmetic
+    of the grouped form, but plain vendor GEMMs of any element type -- the fp32 path, and shapes the grouped kernels refuse."""
+    E, F, K = w_up.shape
+    from semi_pd_amd.layers.basic import dense_linear
+    u = dense_linear(hidden_states, w_up.view(E * F, K))
+    ops.routed_relu_square_(u, topk_weights, topk_ids, E)
+    return dense_linear(u, w_down_cat)
+
+
+class UngatedMoE(nn.Module):
+    """Mixture of two-layer feed-forward experts without a gate branch: softmax over all router logits (fp32), the top_k
+    largest kept and divided by their sum, experts down(act(up(x))), activation "relu2" = squared ReLU.  One GPU per
+    replica.  The router weight is kept in fp32 and multiplied in fp32 (its input is the activation-type rows)."""
+
+    def __init__(self, num_experts: int, top_k: int, hidden_size: int, intermediate_size: int, activation: str = "relu2",
+                 params_dtype=None):
+        super().__init__()
+        if activation not in UNGATED_ACTIVATIONS:
+            raise ValueError(f"UngatedMoE: activation {activation!r} is not supported ({sorted(UNGATED_ACTIVATIONS)})")
+        if not 0 < top_k <= num_experts:
+            raise ValueError(f"UngatedMoE: top {top_k} of {num_experts} experts")
+        self.num_experts, self.top_k, self.activation = num_experts, top_k, activation
+        self.router = nn.Parameter(torch.empty(num_experts, hidden_size, dtype=torch.float32), requires_grad=False)
+        self.w_up = nn.Parameter(torch.empty(num_experts, intermediate_size, hidden_size, dtype=params_dtype), requires_grad=False)
+        self.w_down = nn.Parameter(torch.empty(num_experts, hidden_size, intermediate_size, dtype=params_dtype), requires_grad=False)
+        self.w_down_cat: Optional[torch.Tensor] = None
+
+    def side_by_side(self) -> bool:
+        """fp32 models (the grouped kernels are 16-bit) and SEMIPD_MOE_SIDE_BY_SIDE=1 (A/B knob)."""
+        return self.w_up.dtype == torch.float32 or os.environ.get("SEMIPD_MOE_SIDE_BY_SIDE") == "1"
+
+    def post_load_weights(self):
+        if self.side_by_side():
+            E, K, F = self.w_down.shape
+            self.w_down_cat = self.w_down.permute(1, 0, 2).reshape(K, E * F).contiguous()
+
+    def route(self, hidden_states: torch.Tensor):
+        logits = torch.mm(hidden_states.float(), self.router.t())
+        return ops.topk_softmax(logits, self.top_k, True)
+
+    def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
+        topk_weights, topk_ids = self.route(hidden_states)
+        if self.w_down_cat is not None:
+            return side_by_side_experts(hidden_states, self.w_up, self.w_down_cat, topk_weights, topk_ids)
+        return fused_experts_ungated(hidden_states, self.w_up, self.w_down, topk_weights, topk_ids, self.activation)

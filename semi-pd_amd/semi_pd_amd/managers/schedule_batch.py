@@ -40,6 +40,9 @@ class Req:
         # host mirror of this request's row of req_to_token, kept by the side that allocates (the decode instance,
         # or the unified scheduler): frees never read the device table
         self.kv_slots: List[int] = []
+        # row of the recurrent-state pool (models with recurrent layers; mem_cache/memory_pool.py: RecurrentStatePool).  Unlike
+        # the row of req_to_token it stays with the request between the portions of a chunked prompt
+        self.state_slot: Optional[int] = None
         self.extend_input_len = 0
         self.is_chunked = 0
         self.is_retracted = is_retracted
@@ -79,6 +82,7 @@ class Req:
         self.extend_input_len = 0
         self.is_retracted = True
         self.req_pool_idx = None
+        self.state_slot = None
         self.is_chunked = 0
 
 
@@ -86,11 +90,18 @@ class ChunkCache:
     """mem_cache/chunk_cache.py: no prefix sharing; keeps the KV indices of an unfinished (chunked)
     request and frees everything when a request finishes."""
 
-    def __init__(self, req_to_token_pool, token_to_kv_pool_allocator):
+    def __init__(self, req_to_token_pool, token_to_kv_pool_allocator, state_pool=None):
         self.req_to_token_pool = req_to_token_pool
         self.token_to_kv_pool_allocator = token_to_kv_pool_allocator
+        self.state_pool = state_pool          # RecurrentStatePool of models with recurrent layers, else None
+
+    def release_state(self, req: Req):
+        if req.state_slot is not None:
+            self.state_pool.free(req.state_slot)
+            req.state_slot = None
 
     def cache_finished_req(self, req: Req):
+        self.release_state(req)
         # KV exists for every token but the last sampled one; a slot taken for a step that runs beyond the end of
         # the request (overlapped decode loop) stays in req.kv_slots and is released when that step is processed
         n = len(req.origin_input_ids) + len(req.output_ids) - 1
@@ -108,6 +119,7 @@ class ChunkCache:
         if req.req_pool_idx is not None:
             self.req_to_token_pool.free(req.req_pool_idx)
             req.req_pool_idx = None
+        self.release_state(req)
         self.token_to_kv_pool_allocator.free(req.kv_slots)
         req.kv_slots = []
         req.prefix_indices = torch.empty(0, dtype=torch.int64)
@@ -131,6 +143,7 @@ class ModelWorkerBatch:
     return_logprob: bool = False
     top_logprobs_nums: Optional[List[int]] = None
     extend_logit_rows: Optional[torch.Tensor] = None   # see ForwardBatch.extend_logit_rows
+    state_indices: Optional[torch.Tensor] = None       # int64 [B]: rows of the recurrent-state pool (None: no such pool)
 
 
 def host_list_to_device(values, dtype, device) -> torch.Tensor:
@@ -159,6 +172,7 @@ class ScheduleBatch:
         self.prefix_lens = self.extend_lens = None
         self.extend_num_tokens = 0
         self.decoding_reqs = None
+        self.state_indices: Optional[torch.Tensor] = None
 
     @classmethod
     def init_new(cls, reqs, req_to_token_pool, token_to_kv_pool_allocator, tree_cache, device):
@@ -176,6 +190,22 @@ class ScheduleBatch:
         if idx is None:
             raise RuntimeError("Out of memory. Please set a smaller number for `--max-running-requests`.")
         return idx
+
+    def alloc_state_slots(self):
+        """Models with recurrent layers: every request of the batch holds a row of the state pool from its first portion to
+        its end; the batch carries the rows as a device tensor."""
+        pool = getattr(self.tree_cache, "state_pool", None)
+        if pool is None:
+            self.state_indices = None
+            return
+        for r in self.reqs:
+            if r.state_slot is None:
+                if len(r.prefix_indices):
+                    raise RuntimeError(f"request {r.rid} continues a sequence whose recurrent state was given up")
+                r.state_slot = pool.alloc()
+                if r.state_slot is None:
+                    raise RuntimeError("Out of recurrent-state slots. Please set a smaller number for `--max-running-requests`.")
+        self.state_indices = host_list_to_device([r.state_slot for r in self.reqs], torch.int64, self.device)
 
     def alloc_token_slots(self, num_tokens: int) -> torch.Tensor:
         out = self.token_to_kv_pool_allocator.alloc(num_tokens)
@@ -208,6 +238,7 @@ class ScheduleBatch:
         table = self.req_to_token_pool.req_to_token
         for r, idx in zip(reqs, req_pool_indices):
             r.req_pool_idx = idx
+        self.alloc_state_slots()
         if pre_allocated_req_pool_indices is None:
             # decode instance: the only allocator.  Writes the *shared* table.
             out_cpu = self.alloc_token_slots(extend_num_tokens)
@@ -256,6 +287,7 @@ class ScheduleBatch:
             n = len(req.origin_input_ids) + len(req.output_ids) - 1
             self.token_to_kv_pool_allocator.free(req.kv_slots[:n])
             self.req_to_token_pool.free(req.req_pool_idx)
+            self.tree_cache.release_state(req)
             req.reset_for_retract()
         self.filter_batch(keep_indices=sorted(order))
         total_decoded = sum(len(r.output_ids) for r in self.reqs)
@@ -275,6 +307,8 @@ class ScheduleBatch:
         # req_to_token[req, seq_len] = new slot; then seq_len += 1 (schedule_batch.py:1190-1205)
         self.req_to_token_pool.req_to_token[self.req_pool_indices, self.seq_lens] = self.out_cache_loc.to(torch.int32)
         self.seq_lens = self.seq_lens + 1
+        if getattr(self.tree_cache, "state_pool", None) is not None:
+            self.state_indices = host_list_to_device([r.state_slot for r in self.reqs], torch.int64, self.device)
         self.seq_lens_sum += bs
         self.seq_lens_cpu = [x + 1 for x in self.seq_lens_cpu]
 
@@ -320,7 +354,8 @@ class ScheduleBatch:
             sampling_info=SamplingBatchInfo.from_reqs(self.reqs, getattr(self, "vocab_size", 0), self.device),
             return_logprob=any(r.return_logprob for r in self.reqs),
             top_logprobs_nums=[r.top_logprobs_num if r.return_logprob else 0 for r in self.reqs],
-            extend_logit_rows=getattr(self, "extend_logit_rows", None) if ext else None)
+            extend_logit_rows=getattr(self, "extend_logit_rows", None) if ext else None,
+            state_indices=self.state_indices)
 
 
 class AddReqResult(Enum):

@@ -270,3 +270,53 @@ class MLATokenToKVPool:
     def set_kv_buffer(self, layer, loc: torch.Tensor, cache_k: torch.Tensor, cache_v: torch.Tensor = None):
         ops.store_kv_rows(self.kv_buffer[layer.layer_id], loc,
                           cache_k.view(-1, 1, self.kv_lora_rank + self.qk_rope_head_dim))
+
+
+class RecurrentStatePool:
+    """Per-request state rows of recurrent layers: ONE fp32 slab state[size + 1, sum of widths], every recurrent layer a
+    column range of it (`get_state_buffer(i)`: a [size + 1, width_i] view whose row stride is the slab's), so a request's
+    whole recurrent state is one row and one slot index serves every layer.  Row 0 is the dummy row that padded entries of
+    a captured decode batch read and write, like slot 0 of the KV pools; slots 1 .. size are handed out by a FIFO free
+    list with an in-use bitmap (releasing a slot twice raises).  A slot is not cleared when it changes hands: the kernels
+    start a sequence from zero themselves when a request's first rows arrive (csrc/recurrent.hip), whatever the slot holds.
+    The state keeps fp32 whatever the activation type."""
+
+    def __init__(self, size: int, widths, device: str, bypass_create_buffers: bool = False):
+        self.size = int(size)
+        self.widths = [int(w) for w in widths]
+        self.device = device
+        self.offsets, off = [], 0
+        for w in self.widths:
+            self.offsets.append(off)
+            off += -(-w // 4) * 4              # every range starts on a 16-byte boundary
+        self.row_width = max(off, 4)
+        self.slab: Optional[torch.Tensor] = None
+        self.buffers: List[torch.Tensor] = []
+        if not bypass_create_buffers:
+            self.slab = ipc_safe_zeros((self.size + 1, self.row_width), torch.float32, device)
+            self.buffers = [self.slab[:, o: o + w] for o, w in zip(self.offsets, self.widths)]
+        self.clear()
+
+    def clear(self):
+        self._free = collections.deque(range(1, self.size + 1))
+        self._in_use = bytearray(self.size + 1)
+
+    def available_size(self) -> int:
+        return len(self._free)
+
+    def alloc(self) -> Optional[int]:
+        if not self._free:
+            return None
+        i = self._free.popleft()
+        self._in_use[i] = 1
+        return i
+
+    def free(self, slot: int):
+        slot = int(slot)
+        if not (1 <= slot <= self.size) or not self._in_use[slot]:
+            raise ValueError(f"RecurrentStatePool.free: state slot {slot} is not allocated")
+        self._in_use[slot] = 0
+        self._free.append(slot)
+
+    def get_state_buffer(self, layer_id: int) -> torch.Tensor:
+        return self.buffers[layer_id]

@@ -44,6 +44,9 @@ class ForwardBatch:
     extend_seq_lens_cpu: Optional[List[int]] = None
     extend_prefix_lens_cpu: Optional[List[int]] = None
     extend_logit_rows: Optional[torch.Tensor] = None   # int64 rows of the flat token axis whose logits are wanted (None: last)
+    # recurrent layers: the pool of per-request state rows and each request's row (int64 [B])
+    state_pool: object = None
+    state_indices: Optional[torch.Tensor] = None
     # pools / backend
     req_to_token_pool: object = None
     token_to_kv_pool: object = None
@@ -82,6 +85,10 @@ class ForwardBatch:
         ret.req_to_token_pool = model_runner.req_to_token_pool
         ret.token_to_kv_pool = model_runner.token_to_kv_pool
         ret.attn_backend = model_runner.attn_backend
+        ret.state_pool = getattr(model_runner, "state_pool", None)
+        ret.state_indices = getattr(batch, "state_indices", None)
+        if ret.state_pool is not None and ret.state_indices is None:
+            raise RuntimeError("a model with recurrent layers needs a state row per request (ModelWorkerBatch.state_indices)")
         ret.sampling_info = getattr(batch, "sampling_info", None)
         ret.return_logprob = bool(getattr(batch, "return_logprob", False))
         ret.top_logprobs_nums = getattr(batch, "top_logprobs_nums", None)

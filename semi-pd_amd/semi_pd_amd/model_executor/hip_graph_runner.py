@@ -80,6 +80,8 @@ class HipGraphRunner:
             self.seq_lens = torch.full((self.max_bs,), self.seq_len_fill_value, dtype=torch.int64)
             self.out_cache_loc = torch.zeros(self.max_bs, dtype=torch.int64)
             self.positions = torch.zeros(self.max_bs, dtype=torch.int64)
+            # rows of the recurrent-state pool (row 0, the dummy row, for padded entries)
+            self.state_indices = torch.zeros(self.max_bs, dtype=torch.int64)
         model_runner.attn_backend.init_cuda_graph_state(self.max_bs)
         self.graphs: Dict[Tuple[int, int], torch.cuda.CUDAGraph] = {}      # (CUs of the stream, batch size) -> graph
         self.outputs: Dict[Tuple[int, int], Tuple[torch.Tensor, torch.Tensor]] = {}
@@ -118,7 +120,8 @@ class HipGraphRunner:
             req_pool_indices=self.req_pool_indices[:bs], seq_lens=self.seq_lens[:bs],
             out_cache_loc=self.out_cache_loc[:bs], seq_lens_sum=bs, positions=self.positions[:bs],
             req_to_token_pool=mr.req_to_token_pool, token_to_kv_pool=mr.token_to_kv_pool,
-            attn_backend=mr.attn_backend)
+            attn_backend=mr.attn_backend, state_pool=getattr(mr, "state_pool", None),
+            state_indices=self.state_indices[:bs] if getattr(mr, "state_pool", None) is not None else None)
 
         def run_once():
             torch.clamp(self.seq_lens[:bs] - 1, min=0, out=self.positions[:bs])
@@ -166,6 +169,9 @@ class HipGraphRunner:
             self.seq_lens.fill_(self.seq_len_fill_value)
             self.out_cache_loc.zero_()
             self.req_pool_indices.zero_()
+            self.state_indices.zero_()
+        if forward_batch.state_indices is not None:
+            self.state_indices[:raw_bs].copy_(forward_batch.state_indices)
         self.input_ids[:raw_bs].copy_(forward_batch.input_ids)
         self.req_pool_indices[:raw_bs].copy_(forward_batch.req_pool_indices)
         self.seq_lens[:raw_bs].copy_(forward_batch.seq_lens)

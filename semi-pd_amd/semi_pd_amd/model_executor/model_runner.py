@@ -25,7 +25,7 @@ from semi_pd_amd.distributed import (get_tensor_model_parallel_rank, get_tensor_
                                      init_distributed_environment)
 from semi_pd_amd.layers.attention_backend import HipAttnBackend
 from semi_pd_amd.layers.basic import Sampler
-from semi_pd_amd.mem_cache.memory_pool import (MHATokenToKVPool, MLATokenToKVPool, ReqToTokenPool,
+from semi_pd_amd.mem_cache.memory_pool import (MHATokenToKVPool, MLATokenToKVPool, RecurrentStatePool, ReqToTokenPool,
                                                TokenToKVPoolAllocator)
 from semi_pd_amd.model_executor.forward_batch_info import ForwardBatch, ForwardMode
 from semi_pd_amd.semi_pd.utils import (InstanceRole, IPCInfo, convert_ipc_handle_to_tensor, get_device_sm_count,
@@ -48,6 +48,9 @@ def build_model(model_config, dtype):
     if arch == "Kudirax":
         from semi_pd_amd.models.kudirax import KudiraxForCausalLM
         return KudiraxForCausalLM(model_config, dtype)
+    if arch == "Tigotar":
+        from semi_pd_amd.models.tigotar import TigotarForCausalLM
+        return TigotarForCausalLM(model_config, dtype)
     raise ValueError(f"unsupported architecture {arch}")
 
 
@@ -89,6 +92,8 @@ def dummy_init_weights(model: nn.Module, device: torch.device, seed: int = 0, st
             p.fill_(1.0)
         elif "norm" in leaf and name.endswith("bias"):
             p.zero_()
+        elif "norm" in leaf and name.endswith("alpha"):
+            p.fill_(1.0)      # (the slope of a squashing that stands in for a norm)
         else:
             g = torch.Generator(device=device)
             g.manual_seed(_seed_of(name, seed))
@@ -320,6 +325,15 @@ class ModelRunner:
                                                      dev, bypass_create_buffers=bypass, v_head_dim=geo["v_head_dim"])
         self.token_to_kv_pool_allocator = TokenToKVPoolAllocator(self.max_total_num_tokens, self.kv_cache_dtype, dev,
                                                                  self.token_to_kv_pool)
+        # models with recurrent layers: one fp32 state row per running request (`state_geometry`: the width of every
+        # recurrent layer, in the order of their state ids)
+        self.state_pool = None
+        widths = getattr(self.model, "state_geometry", None)
+        if widths:
+            if self.instance_role != InstanceRole.OTHER:
+                raise ValueError("models with recurrent layers run in the unified engine only: the Semi-PD instances share "
+                                 "the KV pools and the request table between processes, not a state pool")
+            self.state_pool = RecurrentStatePool(self.max_running_requests, widths, dev)
 
     # ------------------------------------------------------------------------------------ IPC export
     @torch.no_grad()

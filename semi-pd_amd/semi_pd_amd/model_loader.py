@@ -27,7 +27,8 @@ def _config_classes():
     from semi_pd_amd.models.llama import LlamaConfig
     from semi_pd_amd.models.kudirax import KudiraxConfig
     from semi_pd_amd.models.opt import OPTConfig
-    return {"LlamaForCausalLM": LlamaConfig, "OPTForCausalLM": OPTConfig,
+    from semi_pd_amd.models.tigotar import TigotarConfig
+    return {"Tigotar": TigotarConfig, "LlamaForCausalLM": LlamaConfig, "OPTForCausalLM": OPTConfig,
             "DeepseekV2ForCausalLM": DeepseekV2Config, "DeepseekV3ForCausalLM": DeepseekV2Config,
             "Kudirax": KudiraxConfig}
 
@@ -143,6 +144,66 @@ def _kudirax_items(config, weights):
         raise RuntimeError(f"checkpoint ended with incomplete stacked parameters: {list(st.pending)[:4]}")
 
 
+_TIGOTAR_RE = re.compile(r"^l(\d+)\.(mix|mlp|norm1b|norm2b|norm1|norm2)(?:\.(.+))?$")
+_TIGOTAR_IN = {"left.q": 0, "left.k": 1, "left.v": 2, "right.z": 3, "right.x": 4, "right.g": 5}
+_TIGOTAR_OUT = {"left.o": 0, "right.o": 1}
+_TIGOTAR_BIAS = {"left.q.b": "bias_q", "left.k.b": "bias_k", "left.v.b": "bias_v", "right.z.b": "bias_z", "right.x.b": "bias_x",
+                 "left.pb": "head_bias"}
+_DYN_TANH_LEAF = {None: "weight", "b": "bias", "alpha": "alpha"}
+
+
+def _tigotar_items(config, weights):
+    """Tigotar checkpoint names (embed, embed.norm[.b|.alpha], loop.in, loop.step, l<i>.norm1[b][.b|.alpha], l<i>.mix.left.q[.b]
+    ..., l<i>.mix.right.z[.b] ..., l<i>.mlp.router, l<i>.mlp.e<j>.up|down, final.norm..., head) -> product parameters:
+    q | k | v | z | x | g stack into the mixer's merged input projection, left.o | right.o side by side into its output
+    projection, the experts' matrices into [E, ...] stacks."""
+    st = _Stacker()
+    top = {"embed": "embed.weight", "head": "head.weight", "loop.in": "loop_in.weight", "loop.step": "loop_step"}
+    for name, t in weights:
+        if name in top:
+            if name.startswith("loop.") and not config.has_loop:
+                continue                      # nothing is repeated: the pass entry does not exist
+            yield top[name], t
+            continue
+        m = re.match(r"^(embed|final)\.norm(?:\.(b|alpha))?$", name)
+        if m:
+            yield f"{m.group(1)}_norm." + _DYN_TANH_LEAF[m.group(2)], t
+            continue
+        m = _TIGOTAR_RE.match(name)
+        if not m or int(m.group(1)) >= len(config.layers):
+            raise KeyError(f"checkpoint tensor {name} has no counterpart in a Tigotar model")
+        i, part, leaf = int(m.group(1)), m.group(2), m.group(3)
+        base = f"layers.{i}."
+        lc = config.layers[i]
+        if part.startswith("norm"):
+            if part in ("norm2", "norm2b") and not lc.experts:
+                continue                      # a layer without feed-forward has no second pair of squashings to apply
+            if leaf not in _DYN_TANH_LEAF:
+                raise KeyError(f"checkpoint tensor {name} has no counterpart in a Tigotar model")
+            yield base + part + "." + _DYN_TANH_LEAF[leaf], t
+        elif part == "mix":
+            if leaf in _TIGOTAR_IN:
+                yield from st.add(base + "mix.in_proj.weight", _TIGOTAR_IN[leaf], 6, t)
+            elif leaf in _TIGOTAR_OUT:
+                yield from st.add(base + "mix.out_proj.weight", _TIGOTAR_OUT[leaf], 2, t, dim=1)
+            elif leaf in _TIGOTAR_BIAS:
+                yield base + "mix." + _TIGOTAR_BIAS[leaf], t
+            else:
+                raise KeyError(f"checkpoint tensor {name} has no counterpart in a Tigotar model")
+        else:
+            if not lc.experts:
+                raise KeyError(f"checkpoint tensor {name}: layer {i} has no feed-forward")
+            if leaf == "router":
+                yield base + "mlp.router", t
+                continue
+            em = re.match(r"^e(\d+)\.(up|down)$", leaf or "")
+            if not em or int(em.group(1)) >= lc.experts:
+                raise KeyError(f"checkpoint tensor {name} has no counterpart in a Tigotar model")
+            yield from st.add(base + "mlp.w_" + em.group(2), int(em.group(1)), lc.experts, t, dim=None)
+    if st.pending:
+        raise RuntimeError(f"checkpoint ended with incomplete stacked parameters: {list(st.pending)[:4]}")
+
+
 _EXPERT_RE = re.compile(r"^(.*\.mlp\.experts)\.(\d+)\.(gate_proj|up_proj|down_proj)\.(weight|weight_scale_inv)$")
 
 
@@ -151,6 +212,9 @@ def product_items(config, weights: Iterable[Tuple[str, torch.Tensor]]) -> Iterat
     arch = config.architectures[0]
     if arch == "Kudirax":
         yield from _kudirax_items(config, weights)
+        return
+    if arch == "Tigotar":
+        yield from _tigotar_items(config, weights)
         return
     st = _Stacker()
     tie = bool(getattr(config, "tie_word_embeddings", False))

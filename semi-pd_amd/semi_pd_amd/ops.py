@@ -1402,3 +1402,163 @@ def bias_relu_square_(u: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Te
     check(lib.semipd_bias_relu_square(ptr(u), u.stride(0), ptr(bias), u.shape[0], u.shape[1], dtype_code(u.dtype),
                                       current_stream(u.device)), "bias_relu_square")
     return u
+
+
+# ---- dynamic tanh, window attention with sigmoid weights, minGRU, routed squared ReLU ------------------------------------
+def dyn_tanh(x: Optional[torch.Tensor], params_in, residual: Optional[torch.Tensor] = None, accumulate: bool = True,
+             params_out=None, want_out: bool = True, out_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """tanh(alpha x) * weight + bias around an fp32 residual stream (csrc/layernorm.hip: semipd_dyn_tanh).
+    params_in / params_out: (weight [width], bias [width], alpha [one element]) of the activation type, or None.
+    v = squash_in(x) when x is given (rows fp32 or of the activation type); with `residual` (fp32 [rows, width]):
+    v += residual (accumulate, or no x), residual <- v (x given); returns squash_out(v), or v, in the activation type (None
+    with want_out=False)."""
+    ref = x if x is not None else residual
+    if ref is None or ref.dim() != 2 or ref.stride(1) != 1:
+        raise RuntimeError("dyn_tanh: needs 2-D rows with unit inner stride to read")
+    rows, width = ref.shape
+    some = params_in if params_in is not None else params_out
+    if some is None:
+        raise RuntimeError("dyn_tanh: no parameters at all")
+    dt = some[0].dtype
+    for prm in (params_in, params_out):
+        if prm is not None:
+            w, b, al = prm
+            if w.shape != (width,) or b.shape != (width,) or al.numel() != 1 or w.dtype != dt or b.dtype != dt or al.dtype != dt:
+                raise RuntimeError("dyn_tanh: weight / bias are [width], alpha one element, all of one type")
+    if (x is None) != (params_in is None):
+        raise RuntimeError("dyn_tanh: an input comes with its parameters")
+    if x is not None and x.dtype not in (dt, torch.float32):
+        raise RuntimeError("dyn_tanh: input rows are fp32 or of the parameters' type")
+    if residual is not None and (residual.dtype != torch.float32 or residual.shape != (rows, width) or residual.stride(1) != 1):
+        raise RuntimeError("dyn_tanh: residual is fp32 [rows, width]")
+    if out_dtype is not None and out_dtype != dt:
+        raise RuntimeError("dyn_tanh: the output has the parameters' type")
+    out = torch.empty((rows, width), dtype=dt, device=ref.device) if (want_out or residual is None) else None
+    pi, po = params_in or (None, None, None), params_out or (None, None, None)
+    lib = _lib.load()
+    check(lib.semipd_dyn_tanh(ptr(x), x.stride(0) if x is not None else 0,
+                              1 if (x is not None and x.dtype == torch.float32 and dt != torch.float32) else 0,
+                              ptr(pi[0]), ptr(pi[1]), ptr(pi[2]), ptr(residual), residual.stride(0) if residual is not None else 0,
+                              1 if accumulate else 0, ptr(po[0]), ptr(po[1]), ptr(po[2]), ptr(out),
+                              out.stride(0) if out is not None else 0, rows, width, dtype_code(dt), current_stream(ref.device)),
+          "dyn_tanh")
+    return out
+
+
+def routed_relu_square_(u: torch.Tensor, topk_weights: torch.Tensor, topk_ids: torch.Tensor, num_experts: int) -> torch.Tensor:
+    """u [T, experts * ff] in place: relu(u)^2 times the routing weight of the column's expert for the row's token (0 for
+    experts the token does not use) (csrc/layernorm.hip)."""
+    T, width = u.shape
+    if u.stride(1) != 1 or width % num_experts or topk_weights.dtype != torch.float32 or topk_ids.dtype != torch.int32 \
+            or topk_weights.shape != topk_ids.shape or topk_ids.shape[0] != T or not topk_weights.is_contiguous() \
+            or not topk_ids.is_contiguous():
+        raise RuntimeError("routed_relu_square_: u [T, experts * ff], topk_weights fp32 / topk_ids int32 [T, k] contiguous")
+    lib = _lib.load()
+    check(lib.semipd_routed_relu_square(ptr(u), u.stride(0), ptr(topk_weights), ptr(topk_ids), topk_ids.shape[1], T,
+                                        width // num_experts, num_experts, dtype_code(u.dtype), current_stream(u.device)),
+          "routed_relu_square")
+    return u
+
+
+def min_gru(proj: torch.Tensor, z_off: int, x_off: int, g_off: int, width: int, bias_z: Optional[torch.Tensor],
+            bias_x: Optional[torch.Tensor], out: torch.Tensor, state: torch.Tensor, state_indices: torch.Tensor,
+            seq_lens: torch.Tensor, q_start: Optional[torch.Tensor], q_len: Optional[torch.Tensor], max_q_len: int,
+            out_scale: float = 1.0) -> None:
+    """minGRU over the rows of `proj` (columns z | x | g at the given offsets, `width` each) with the per-request fp32 state
+    rows state[state_indices[b]] (csrc/recurrent.hip): out [T, width] (may be a column range) <- out_scale * S * silu(g)."""
+    T = proj.shape[0]
+    B = state_indices.shape[0]
+    if proj.dim() != 2 or proj.stride(1) != 1 or out.dim() != 2 or out.stride(1) != 1 or out.shape != (T, width) \
+            or out.dtype != proj.dtype:
+        raise RuntimeError("min_gru: proj / out are 2-D rows of one type, out [T, width]")
+    if state.dtype != torch.float32 or state.dim() != 2 or state.shape[1] != width or state.stride(1) != 1:
+        raise RuntimeError("min_gru: state is fp32 [slots, width]")
+    if state_indices.dtype != torch.int64 or seq_lens.dtype != torch.int64 or seq_lens.shape[0] != B:
+        raise RuntimeError("min_gru: state_indices / seq_lens are int64 [B]")
+    for b_ in (bias_z, bias_x):
+        if b_ is not None and (b_.shape != (width,) or b_.dtype != proj.dtype):
+            raise RuntimeError("min_gru: biases are [width] of the activation type")
+    if (q_start is None) != (q_len is None) or (q_start is None and T != B):
+        raise RuntimeError("min_gru: q_start and q_len come together; without them one row per request")
+    if q_start is not None and (q_start.dtype != torch.int32 or q_len.dtype != torch.int32 or q_start.shape[0] != B
+                                or q_len.shape[0] != B):
+        raise RuntimeError("min_gru: q_start / q_len are int32 [B]")
+    lib = _lib.load()
+    work, nbytes = None, 0
+    if q_start is not None and max_q_len > 256:
+        nbytes = int(lib.semipd_min_gru_workspace(T, B, width))
+        work = torch.empty(nbytes // 4, dtype=torch.float32, device=proj.device)
+    check(lib.semipd_min_gru(ptr(proj), proj.stride(0), z_off, x_off, g_off, ptr(bias_z), ptr(bias_x), ptr(out), out.stride(0),
+                             ptr(state), state.stride(0), ptr(state_indices), ptr(seq_lens), ptr(q_start), ptr(q_len), B, T,
+                             int(max_q_len), width, float(out_scale), ptr(work), nbytes, dtype_code(proj.dtype),
+                             current_stream(proj.device)), "min_gru")
+
+
+def bias_rope_vnorm_kv_store(qkv: torch.Tensor, num_q_heads: int, num_kv_heads: int, qk_dim: int, v_dim: int, k_off: int,
+                             v_off: int, bias_q: Optional[torch.Tensor], bias_k: Optional[torch.Tensor],
+                             bias_v: Optional[torch.Tensor], positions: torch.Tensor, inv_freq: Optional[torch.Tensor],
+                             rot_dims: int, eps: float, k_buffer: torch.Tensor, v_buffer: torch.Tensor, loc: torch.Tensor) -> None:
+    """Rows of `qkv` hold q | k | v at columns 0, k_off, v_off: + biases, neighbouring pairs of the first rot_dims elements of
+    every q / k head turned by positions * inv_freq, values to unit RMS; q in place, k / v into the pools at `loc`
+    (csrc/local_attention.hip)."""
+    if qkv.dim() != 2 or qkv.stride(1) != 1:
+        raise RuntimeError("bias_rope_vnorm_kv_store: qkv must be 2-D with contiguous rows")
+    T = qkv.shape[0]
+    if loc.dtype != torch.int64 or positions.dtype != torch.int64 or loc.shape[0] != T or positions.shape[0] != T:
+        raise RuntimeError("bias_rope_vnorm_kv_store: one int64 pool slot and position per row")
+    for buf, size, name in ((k_buffer, qk_dim, "k_buffer"), (v_buffer, v_dim, "v_buffer")):
+        if buf.dtype != qkv.dtype or buf.dim() != 3 or buf.shape[1] != num_kv_heads or buf.shape[2] != size \
+                or not buf.is_contiguous():
+            raise RuntimeError(f"bias_rope_vnorm_kv_store: {name} must be a contiguous [N, {num_kv_heads}, {size}] pool of "
+                               f"{qkv.dtype}, got {tuple(buf.shape)} {buf.dtype}")
+    for b_, n in ((bias_q, num_q_heads * qk_dim), (bias_k, num_kv_heads * qk_dim), (bias_v, num_kv_heads * v_dim)):
+        if b_ is not None and (b_.shape != (n,) or b_.dtype != qkv.dtype or not b_.is_contiguous()):
+            raise RuntimeError("bias_rope_vnorm_kv_store: biases are contiguous [heads * size] of the activation type")
+    if rot_dims and (inv_freq is None or inv_freq.dtype != torch.float32 or inv_freq.numel() != rot_dims // 2
+                     or not inv_freq.is_contiguous()):
+        raise RuntimeError("bias_rope_vnorm_kv_store: inv_freq is fp32 [rot_dims / 2]")
+    if qkv.shape[1] < v_off + num_kv_heads * v_dim:
+        raise RuntimeError("bias_rope_vnorm_kv_store: rows too short for the column offsets")
+    lib = _lib.load()
+    check(lib.semipd_bias_rope_vnorm_kv_store(ptr(qkv), qkv.stride(0), T, num_q_heads, num_kv_heads, qk_dim, v_dim, k_off, v_off,
+                                              ptr(bias_q), ptr(bias_k), ptr(bias_v), ptr(positions), ptr(inv_freq), int(rot_dims),
+                                              float(eps), ptr(k_buffer), ptr(v_buffer), ptr(loc), dtype_code(qkv.dtype),
+                                              current_stream(qkv.device)), "bias_rope_vnorm_kv_store")
+
+
+def window_attention_fwd(q: torch.Tensor, out: torch.Tensor, k_buffer: torch.Tensor, v_buffer: torch.Tensor,
+                         req_to_token: torch.Tensor, req_pool_indices: torch.Tensor, seq_lens: torch.Tensor,
+                         q_start: Optional[torch.Tensor], q_len: Optional[torch.Tensor], max_q_len: int, sm_scale: float,
+                         window: int = 0, keep_first: int = 0, head_bias: Optional[torch.Tensor] = None, sigmoid: bool = False,
+                         sink: Optional[torch.Tensor] = None, out_scale: float = 1.0, form: int = 0) -> None:
+    """Attention over the paged pools with a sliding window that keeps the first positions of the sequence visible, and
+    optionally independent sigmoid weights (csrc/local_attention.hip: semipd_window_attention).  Batch description as in
+    local_attention_fwd.  A query at position p sees key j <= p when p - j < window (0: no limit) or j < keep_first;
+    sigmoid: weight = sigmoid(sm_scale * q.k + head_bias[head]), no normalisation; else softmax (+ sink)."""
+    T = q.shape[0]
+    G, D = k_buffer.shape[1], k_buffer.shape[2]
+    E = v_buffer.shape[2]
+    if q.dim() != 2 or out.dim() != 2 or q.stride(1) != 1 or out.stride(1) != 1 or q.shape[1] % D or out.shape[1] % E:
+        raise RuntimeError("window_attention_fwd: q / out are [T, heads * size] with contiguous rows")
+    H = q.shape[1] // D
+    if out.shape != (T, H * E) or out.dtype != q.dtype or k_buffer.dtype != q.dtype or v_buffer.dtype != q.dtype:
+        raise RuntimeError("window_attention_fwd: shapes or types of q, out and the pools disagree")
+    if not (k_buffer.is_contiguous() and v_buffer.is_contiguous()) or v_buffer.shape[1] != G:
+        raise RuntimeError("window_attention_fwd: pools must be contiguous [N, G, size]")
+    for vec, name in ((head_bias, "head_bias"), (sink, "sink")):
+        if vec is not None and (vec.dtype != torch.float32 or vec.numel() != H or not vec.is_contiguous()):
+            raise RuntimeError(f"window_attention_fwd: {name} is fp32 [H]")
+    if req_to_token.dtype != torch.int32 or req_pool_indices.dtype != torch.int64 or seq_lens.dtype != torch.int64:
+        raise RuntimeError("window_attention_fwd: req_to_token int32, req_pool_indices / seq_lens int64")
+    B = req_pool_indices.shape[0]
+    if (q_start is None) != (q_len is None) or (q_start is None and T != B):
+        raise RuntimeError("window_attention_fwd: q_start and q_len come together; without them one row per request")
+    if q_start is not None and (q_start.dtype != torch.int32 or q_len.dtype != torch.int32
+                                or q_start.shape[0] != B or q_len.shape[0] != B):
+        raise RuntimeError("window_attention_fwd: q_start / q_len are int32 [B]")
+    lib = _lib.load()
+    check(lib.semipd_window_attention(ptr(q), q.stride(0), ptr(out), out.stride(0), ptr(k_buffer), ptr(v_buffer),
+                                      ptr(req_to_token), req_to_token.stride(0), ptr(req_pool_indices), ptr(seq_lens),
+                                      ptr(q_start), ptr(q_len), B, T, int(max_q_len), H, G, D, E, float(sm_scale), int(window),
+                                      int(keep_first), ptr(head_bias), 1 if sigmoid else 0, ptr(sink), float(out_scale),
+                                      int(form), dtype_code(q.dtype), current_stream(q.device)), "window_attention")
