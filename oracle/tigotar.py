@@ -77,20 +77,26 @@ def window_attention_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], pre: str
     return o.reshape(T, H * E) @ w[pre + "o"].float().T
 
 
-def min_gru_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], pre: str) -> torch.Tensor:
-    """S_t = (1 - z_t) S_(t-1) + z_t c_t from S = 0, gate z and candidate c functions of token t alone; the output is
-    W_o (S_t * silu(W_g h_t))."""
-    h = h.float()
-    z = torch.sigmoid(h @ w[pre + "z"].float().T + w[pre + "z.b"].float())
-    u = h @ w[pre + "x"].float().T + w[pre + "x.b"].float()
+def min_gru_states(z_lin: torch.Tensor, u: torch.Tensor) -> torch.Tensor:
+    """[T, R] pre-activations of the gate and of the candidate -> the states S_1 .. S_T from S_0 = 0:
+    z = sigmoid(z_lin), c = u + 1/2 where u >= 0 else sigmoid(u), S_t = (1 - z_t) S_(t-1) + z_t c_t."""
+    z = torch.sigmoid(z_lin.float())
+    u = u.float()
     cand = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
     S = torch.zeros(z.shape[1])
     states = []
-    for t in range(h.shape[0]):
+    for t in range(z.shape[0]):
         S = (1.0 - z[t]) * S + z[t] * cand[t]
         states.append(S)
+    return torch.stack(states) if states else torch.zeros(0, z.shape[1])
+
+
+def min_gru_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], pre: str) -> torch.Tensor:
+    """Gate and candidate read token t alone; the branch gives W_o (S_t * silu(W_g h_t))."""
+    h = h.float()
+    S = min_gru_states(h @ w[pre + "z"].float().T + w[pre + "z.b"].float(), h @ w[pre + "x"].float().T + w[pre + "x.b"].float())
     g = h @ w[pre + "g"].float().T
-    return (torch.stack(states) * torch.nn.functional.silu(g)) @ w[pre + "o"].float().T
+    return (S * torch.nn.functional.silu(g)) @ w[pre + "o"].float().T
 
 
 def parallel_mixer(h, w, pre: str, m: dict, eps: float) -> torch.Tensor:

@@ -379,11 +379,12 @@ template <int ND> struct KFrags {
 //   in whole rows; a wave on its own takes its K fragments straight from the pool into operand layout.
 //   32 keys per step (64 between one pair of barriers measured slower: the staging registers of 64 rows push the 128 / 128
 //   kernel into scratch).
-template <typename T, int ND, int NE, int NT, bool BLOCK_SYNC, typename Ok, typename Relevant>
+template <typename T, int ND, int NE, int NT, bool BLOCK_SYNC, bool SIG, typename Ok, typename Relevant>
 __device__ __forceinline__ void key_walk(SoftState<NE>& st, const Frag16 (&qf)[ND], int nd, int ne, int E, const T* kp,
                                          int64_t kstride, const T* vp, int64_t vstride, const int32_t* row, int64_t j_begin,
                                          int64_t j_end, int64_t j_step, uint8_t* v_lds, int tid, float scale, float cap, Ok ok,
-                                         Relevant relevant, int r, int g, const int32_t* idx_lds, int64_t idx_base) {
+                                         Relevant relevant, int r, int g, const int32_t* idx_lds, int64_t idx_base,
+                                         float hb = 0.f) {
   constexpr int KS = 32;                          // keys per step
   constexpr int NV = (NE * 2 * KS) / NT;          // 16-byte pieces of V per thread and step, at most
   constexpr int NK = BLOCK_SYNC ? (ND * 4 * KS) / NT : 1;   // the same for K rows that go through LDS
@@ -489,6 +490,13 @@ __device__ __forceinline__ void key_walk(SoftState<NE>& st, const Frag16 (&qf)[N
       sc[i] = ok(ja + i) ? smap(sa[i]) : -INFINITY;
       sc[4 + i] = ok(jb + i) ? smap(sb[i]) : -INFINITY;
     }
+    float p[8];
+    if constexpr (SIG) {
+      // independent weights sigmoid(score + hb) in the base-2 domain (hb comes multiplied by log2 e): no maximum, no sum;
+      // a masked key has score -inf: exp2(+inf) = inf, 1 / inf = 0
+#pragma unroll
+      for (int i = 0; i < 8; ++i) p[i] = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-(sc[i] + hb)));
+    } else {
     float mt = sc[0];
 #pragma unroll
     for (int i = 1; i < 8; ++i) mt = fmaxf(mt, sc[i]);
@@ -506,13 +514,14 @@ __device__ __forceinline__ void key_walk(SoftState<NE>& st, const Frag16 (&qf)[N
           for (int i = 0; i < 4; ++i) st.acc[eb][i] *= alpha;
       st.m = m_new;
     }
-    float p[8], sum = 0.f;
+    float sum = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       p[i] = __builtin_amdgcn_exp2f(sc[i] - m_safe);
       sum += p[i];
     }
     st.l += sum;
+    }
     Frag16 pb;
 #pragma unroll
     for (int i = 0; i < 4; ++i) pb.w[i] = pack2<T>(p[2 * i], p[2 * i + 1]);
@@ -562,7 +571,7 @@ __device__ __forceinline__ void key_walk(SoftState<NE>& st, const Frag16 (&qf)[N
 }
 
 // Prompt portions: 64 query rows of one request and one head per workgroup, 16 per wave.
-template <typename T, int ND, int NE>
+template <typename T, int ND, int NE, bool SIG>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ND <= 4 ? 4 : 1))) local_attention_mfma_kernel(LocalAttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t v_lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
@@ -603,8 +612,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ND <= 
   const int D = a.D, E = a.E, G = a.G, nd = D >> 5, ne = E >> 4;
   const int gk = h / (a.H / G);
   const int64_t qn = a.q_len[b], base_pos = a.seq_lens[b] - qn, t0 = a.q_start[b];
-  const int chunk = a.chunk;
-  auto lo_of = [&](int64_t p) -> int64_t { return chunk > 0 ? (p / chunk) * chunk : 0; };
+  auto lo_of = [&](int64_t p) -> int64_t { return range_lo(a, p); };
+  const int64_t keep = a.window > 0 ? a.keep_first : 0;      // first positions that stay visible in front of the window
   const int64_t blk_last = (q0 + 63 < qn - 1 ? q0 + 63 : qn - 1);
   const int64_t blk_lo = lo_of(base_pos + q0), blk_hi = base_pos + blk_last;
   // this wave's 16 rows
@@ -628,17 +637,25 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ND <= 
 #pragma unroll
   for (int eb = 0; eb < NE; ++eb) st.acc[eb] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int32_t* row = a.req_to_token + a.req_pool_indices[b] * a.r2t_stride;
-  key_walk<T, ND, NE, 256, true>(
+  const float hb = (SIG && a.head_bias) ? a.head_bias[h] * kLog2e : 0.f;
+  // the kept first positions that lie in front of the tile's window range: visible to every row of the tile
+  const int64_t n_first = keep < blk_lo ? keep : blk_lo;
+  if (n_first > 0)
+    key_walk<T, ND, NE, 256, true, SIG>(
+        st, qf, nd, ne, E, (const T*)a.k_pool + (int64_t)gk * D, (int64_t)G * D, (const T*)a.v_pool + (int64_t)gk * E,
+        (int64_t)G * E, row, 0, n_first - 1, 32, v_lds, tid, a.scale, a.cap, [&](int64_t j) { return q_ok && j < n_first; },
+        [&](int64_t) { return wave_on; }, r, g, nullptr, 0, hb);
+  key_walk<T, ND, NE, 256, true, SIG>(
       st, qf, nd, ne, E, (const T*)a.k_pool + (int64_t)gk * D, (int64_t)G * D, (const T*)a.v_pool + (int64_t)gk * E,
       (int64_t)G * E, row, blk_lo, blk_hi, 32, v_lds, tid, a.scale, a.cap,
-      [&](int64_t j) { return q_ok && j >= my_lo && j <= my_pos; },
-      [&](int64_t j0) { return wave_on && j0 + 31 >= w_lo && j0 <= w_hi; }, r, g, nullptr, blk_lo);
+      [&](int64_t j) { return q_ok && j <= my_pos && (j >= my_lo || j < keep); },
+      [&](int64_t j0) { return wave_on && j0 <= w_hi && (j0 + 31 >= w_lo || j0 < keep); }, r, g, nullptr, blk_lo, hb);
   float l = st.l;
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
   if (!wave_on) return;
-  if (a.sink != nullptr) l += __builtin_amdgcn_exp2f(a.sink[h] * kLog2e - st.m);      // (the running maximum is in the base-2 domain)
-  const float inv = q_ok ? 1.0f / l : 0.f;
+  if (!SIG && a.sink != nullptr) l += __builtin_amdgcn_exp2f(a.sink[h] * kLog2e - st.m);      // (the running maximum is in the base-2 domain)
+  const float inv = q_ok ? (SIG ? a.out_scale : a.out_scale / l) : 0.f;
   // Epilogue through LDS (the tiles are free: the walk ends on a barrier): a lane holds 4 value elements of one row per
   // 16-element block -- written out like that, rows would go to memory in 8-byte pieces; the wave lays its 16 x E tile down in
   // LDS and takes it up again in whole 16-byte pieces of consecutive lanes, so the gate is read and the result written in
@@ -676,7 +693,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(ND <= 
 // Decode steps: one workgroup per (request, kv head, group of 16 q heads); the q heads are the 16 columns, the waves
 // take the 32-key steps in turn, each with a V tile of its own, and meet in LDS.
 // (eight waves for head sizes up to 128, four above: the walk's registers at 256 / 256 do not fit eight waves per CU)
-template <typename T, int ND, int NE, int NW>
+template <typename T, int ND, int NE, int NW, bool SIG>
 __global__ void __launch_bounds__(64 * NW) local_attention_decode_kernel(LocalAttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t v_lds[];
   __shared__ float part_ml[NW][2][16];
@@ -690,7 +707,8 @@ __global__ void __launch_bounds__(64 * NW) local_attention_decode_kernel(LocalAt
   const int64_t t = a.q_start ? (int64_t)a.q_start[b] + a.q_len[b] - 1 : b;     // the request's newest row
   const int64_t pos = a.seq_lens[b] - 1;
   if (pos < 0) return;
-  const int64_t lo = a.chunk > 0 ? (pos / a.chunk) * a.chunk : 0;
+  const int64_t lo = range_lo(a, pos), n_first = kept_before(a, lo);
+  const float hb = (SIG && a.head_bias) ? a.head_bias[h] * kLog2e : 0.f;
   Frag16 qf[ND];
   {
     const T* q = (const T*)a.q + t * a.q_ld + (int64_t)h * D;
@@ -699,7 +717,7 @@ __global__ void __launch_bounds__(64 * NW) local_attention_decode_kernel(LocalAt
       if (kk < nd) qf[kk].u = *reinterpret_cast<const uint4*>(q + 32 * kk + 8 * g);
   }
   SoftState<NE> st;
-  st.m = -INFINITY;
+  st.m = SIG ? 0.f : -INFINITY;       // (sigmoid weights need no running maximum: the partial sums merge as they are)
   st.l = 0.f;
 #pragma unroll
   for (int eb = 0; eb < NE; ++eb) st.acc[eb] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -713,10 +731,16 @@ __global__ void __launch_bounds__(64 * NW) local_attention_decode_kernel(LocalAt
     for (int64_t j = lo + tid; j <= pos; j += 64 * NW) idx_lds[j - lo] = row[j];
     __syncthreads();
   }
-  key_walk<T, ND, NE, 64, false>(
+  // the kept first positions in front of the window (none without one), then the range that ends at the query
+  if (n_first > 0)
+    key_walk<T, ND, NE, 64, false, SIG>(
+        st, qf, nd, ne, E, (const T*)a.k_pool + (int64_t)gk * D, (int64_t)G * D, (const T*)a.v_pool + (int64_t)gk * E,
+        (int64_t)G * E, row, (int64_t)32 * wave, n_first - 1, 32 * NW, mine_b, lane, a.scale, a.cap,
+        [&](int64_t j) { return j < n_first; }, [&](int64_t) { return true; }, r, g, nullptr, 0, hb);
+  key_walk<T, ND, NE, 64, false, SIG>(
       st, qf, nd, ne, E, (const T*)a.k_pool + (int64_t)gk * D, (int64_t)G * D, (const T*)a.v_pool + (int64_t)gk * E,
       (int64_t)G * E, row, lo + 32 * wave, pos, 32 * NW, mine_b, lane, a.scale, a.cap, [&](int64_t j) { return j <= pos; },
-      [&](int64_t) { return true; }, r, g, idx_fits ? idx_lds : nullptr, lo);
+      [&](int64_t) { return true; }, r, g, idx_fits ? idx_lds : nullptr, lo, hb);
   float l = st.l;
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
@@ -748,8 +772,8 @@ __global__ void __launch_bounds__(64 * NW) local_attention_decode_kernel(LocalAt
     lt += f[w] * part_ml[w][1][c];
   }
   const int hh = gk * rep + col0 + c;
-  if (a.sink != nullptr) lt += __builtin_amdgcn_exp2f(a.sink[hh] * kLog2e - m);
-  const float inv = 1.0f / lt;
+  if (!SIG && a.sink != nullptr) lt += __builtin_amdgcn_exp2f(a.sink[hh] * kLog2e - m);
+  const float inv = SIG ? a.out_scale : a.out_scale / lt;
   T* o = (T*)a.out + t * a.out_ld + (int64_t)hh * E;
   const T* gt = a.gate ? (const T*)a.gate + t * a.gate_ld + (int64_t)hh * E : nullptr;
   for (int e = slice; e < E; e += 4 * NW) {
@@ -864,51 +888,67 @@ static int launch_local_attention(LocalAttnArgs a, int64_t max_q_len, int form, 
   SEMIPD_CHECK_ARG(q_start != nullptr || num_tokens == batch, SEMIPD_EINVAL, "local_attention: one row per request without q_start");
   SEMIPD_CHECK_ARG(a.cap >= 0.f, SEMIPD_EINVAL, "local_attention: bad cap");
   const bool half = dtype == SEMIPD_BF16 || dtype == SEMIPD_F16;
-  const bool mfma_ok = half && a.window == 0 && !a.sigmoid && a.out_scale == 1.0f && local_mfma_shape_ok(qk_dim, v_dim) && aligned16(q) && q_ld % 8 == 0 && aligned16(k_pool) &&
+  const bool mfma_ok = half && local_mfma_shape_ok(qk_dim, v_dim) && aligned16(q) && q_ld % 8 == 0 && aligned16(k_pool) &&
                        aligned16(v_pool) && aligned16(out) && out_ld % 8 == 0 &&
                        (gate == nullptr || (aligned16(gate) && gate_ld % 8 == 0));
   SEMIPD_CHECK_ARG(form != 2 || mfma_ok, SEMIPD_ESHAPE, "local_attention: the matrix-core forms do not take this shape or type");
   if (form != 1 && mfma_ok) {
     const bool small = qk_dim <= 128 && v_dim <= 128;
     const int tile = 32 * v_tile_row_bytes(v_dim);                       // at most 32 * 576 bytes: below the 64 KB default
+    const bool sig = a.sigmoid != 0;
     if (q_start == nullptr || max_q_len <= 1) {
       const dim3 grid((unsigned)batch, (unsigned)num_kv_heads, (unsigned)((num_q_heads / num_kv_heads + 15) / 16));
       const int merge = v_dim * 17 * 4;
       const int nw = small ? 8 : 4;
       const size_t lds = nw * (size_t)(tile > merge ? tile : merge);      // up to 80 KB: above the 64 KB default
-      if (lds > 65536) {
-        static std::atomic<uint64_t> done[4] = {};
-        const void* fn = dtype == SEMIPD_BF16
-                             ? (small ? (const void*)local_attention_decode_kernel<bf16_t, 4, 8, 8> : (const void*)local_attention_decode_kernel<bf16_t, 8, 16, 4>)
-                             : (small ? (const void*)local_attention_decode_kernel<f16_t, 4, 8, 8> : (const void*)local_attention_decode_kernel<f16_t, 8, 16, 4>);
-        if (ensure_dynamic_lds(fn, lds, done[(dtype == SEMIPD_BF16 ? 0 : 2) + (small ? 0 : 1)], "local_attention")) return SEMIPD_EINVAL;
-      }
+      static std::atomic<uint64_t> done[8] = {};
+      int rc = -1;
+#define SEMIPD_LA_DEC(TT, NDD, NEE, NWW, SS, SLOT)                                                                              \
+  do {                                                                                                                          \
+    if (lds > 65536 && ensure_dynamic_lds((const void*)local_attention_decode_kernel<TT, NDD, NEE, NWW, SS>, lds, done[SLOT],  \
+                                          "local_attention"))                                                                   \
+      return SEMIPD_EINVAL;                                                                                                     \
+    hipLaunchKernelGGL((local_attention_decode_kernel<TT, NDD, NEE, NWW, SS>), grid, dim3(64 * NWW), lds, as_stream(stream), a); \
+    rc = 0;                                                                                                                     \
+  } while (0)
       if (dtype == SEMIPD_BF16) {
-        if (small) hipLaunchKernelGGL((local_attention_decode_kernel<bf16_t, 4, 8, 8>), grid, dim3(512), lds, as_stream(stream), a);
-        else hipLaunchKernelGGL((local_attention_decode_kernel<bf16_t, 8, 16, 4>), grid, dim3(256), lds, as_stream(stream), a);
+        if (small && !sig) SEMIPD_LA_DEC(bf16_t, 4, 8, 8, false, 0);
+        else if (small) SEMIPD_LA_DEC(bf16_t, 4, 8, 8, true, 1);
+        else if (!sig) SEMIPD_LA_DEC(bf16_t, 8, 16, 4, false, 2);
+        else SEMIPD_LA_DEC(bf16_t, 8, 16, 4, true, 3);
       } else {
-        if (small) hipLaunchKernelGGL((local_attention_decode_kernel<f16_t, 4, 8, 8>), grid, dim3(512), lds, as_stream(stream), a);
-        else hipLaunchKernelGGL((local_attention_decode_kernel<f16_t, 8, 16, 4>), grid, dim3(256), lds, as_stream(stream), a);
+        if (small && !sig) SEMIPD_LA_DEC(f16_t, 4, 8, 8, false, 4);
+        else if (small) SEMIPD_LA_DEC(f16_t, 4, 8, 8, true, 5);
+        else if (!sig) SEMIPD_LA_DEC(f16_t, 8, 16, 4, false, 6);
+        else SEMIPD_LA_DEC(f16_t, 8, 16, 4, true, 7);
       }
+#undef SEMIPD_LA_DEC
+      (void)rc;
       return launch_status("local_attention_decode");
     }
     a.n_tiles = (num_tokens + 63) / 64 + batch;
     const dim3 grid((unsigned)((a.n_tiles * num_q_heads + 7) / 8 * 8));
     const size_t tiles = 2 * ((size_t)tile + 32 * (size_t)(qk_dim * 2 + 32));   // two pairs of (32 V rows, 32 K rows): at most 71.7 KB
-    if (tiles > 65536) {
-      static std::atomic<uint64_t> done_bf16{0}, done_f16{0};
-      if (dtype == SEMIPD_BF16
-              ? ensure_dynamic_lds((const void*)local_attention_mfma_kernel<bf16_t, 8, 16>, tiles, done_bf16, "local_attention")
-              : ensure_dynamic_lds((const void*)local_attention_mfma_kernel<f16_t, 8, 16>, tiles, done_f16, "local_attention"))
-        return SEMIPD_EINVAL;
-    }
+    static std::atomic<uint64_t> done_p[8] = {};
+#define SEMIPD_LA_PRE(TT, NDD, NEE, SS, SLOT)                                                                                   \
+  do {                                                                                                                          \
+    if (tiles > 65536 && ensure_dynamic_lds((const void*)local_attention_mfma_kernel<TT, NDD, NEE, SS>, tiles, done_p[SLOT],    \
+                                            "local_attention"))                                                                 \
+      return SEMIPD_EINVAL;                                                                                                     \
+    hipLaunchKernelGGL((local_attention_mfma_kernel<TT, NDD, NEE, SS>), grid, dim3(256), tiles, as_stream(stream), a);           \
+  } while (0)
     if (dtype == SEMIPD_BF16) {
-      if (small) hipLaunchKernelGGL((local_attention_mfma_kernel<bf16_t, 4, 8>), grid, dim3(256), tiles, as_stream(stream), a);
-      else hipLaunchKernelGGL((local_attention_mfma_kernel<bf16_t, 8, 16>), grid, dim3(256), tiles, as_stream(stream), a);
+      if (small && !sig) SEMIPD_LA_PRE(bf16_t, 4, 8, false, 0);
+      else if (small) SEMIPD_LA_PRE(bf16_t, 4, 8, true, 1);
+      else if (!sig) SEMIPD_LA_PRE(bf16_t, 8, 16, false, 2);
+      else SEMIPD_LA_PRE(bf16_t, 8, 16, true, 3);
     } else {
-      if (small) hipLaunchKernelGGL((local_attention_mfma_kernel<f16_t, 4, 8>), grid, dim3(256), tiles, as_stream(stream), a);
-      else hipLaunchKernelGGL((local_attention_mfma_kernel<f16_t, 8, 16>), grid, dim3(256), tiles, as_stream(stream), a);
+      if (small && !sig) SEMIPD_LA_PRE(f16_t, 4, 8, false, 4);
+      else if (small) SEMIPD_LA_PRE(f16_t, 4, 8, true, 5);
+      else if (!sig) SEMIPD_LA_PRE(f16_t, 8, 16, false, 6);
+      else SEMIPD_LA_PRE(f16_t, 8, 16, true, 7);
     }
+#undef SEMIPD_LA_PRE
     return launch_status("local_attention_mfma");
   }
   const dim3 grid((unsigned)((num_tokens + 3) / 4), (unsigned)num_q_heads);

@@ -442,8 +442,10 @@ class UngatedMoE(nn.Module):
         self.w_down_cat: Optional[torch.Tensor] = None
 
     def side_by_side(self) -> bool:
-        """fp32 models (the grouped kernels are 16-bit) and SEMIPD_MOE_SIDE_BY_SIDE=1 (A/B knob)."""
-        return self.w_up.dtype == torch.float32 or os.environ.get("SEMIPD_MOE_SIDE_BY_SIDE") == "1"
+        """fp32 models (the grouped kernels are 16-bit), widths whose rows the kernel that sums a token's experts does not
+        take (16-byte pieces: a multiple of 8), and SEMIPD_MOE_SIDE_BY_SIDE=1 (A/B knob)."""
+        return (self.w_up.dtype == torch.float32 or self.w_up.shape[2] % 8 != 0
+                or os.environ.get("SEMIPD_MOE_SIDE_BY_SIDE") == "1")
 
     def post_load_weights(self):
         if self.side_by_side():
