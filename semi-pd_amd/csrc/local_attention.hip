@@ -3,7 +3,7 @@
 //  * unit_norm_kv_store_kernel: per head, q <- q / rms(q) in place, k <- k / rms(k) into the key pool,
 //    v <- (1 - a) v + a v0 (optional) into the value pool.  Everything between the projection GEMM and the attention
 //    in one launch; sums of squares, the division and the blend in fp32.
-//  * local_attention_rows_kernel: one wave per (query row, head) for every element type, any head sizes up to 512 / 256.
+//  * local_attention_rows_kernel: one wave per (query row, head) for every element type, any head sizes up to 512 / 512.
 //    Keys come from the paged pools through the request's row of req_to_token, so a prompt portion, a whole prompt and
 //    a decode step are the same walk: query at position p sees keys lo(p) .. p, lo(p) = floor(p / chunk) * chunk
 //    (chunk 0: lo = 0).  score = cap * tanh(scale * q.k / cap) (cap 0: none); the softmax denominator holds one more
@@ -163,9 +163,9 @@ __global__ void __launch_bounds__(256) bias_rope_vnorm_kv_store_kernel(
     const int g = h - H - G;
     const T* src = row + v_off + (int64_t)g * E;
     T* dst = v_pool + (loc[t] * G + g) * E;
-    float x[4], ss = 0.f;      // E <= 256
+    float x[8], ss = 0.f;      // E <= 512
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < 8; ++u) {
       const int e = lane + 64 * u;
       x[u] = 0.f;
       if (e < E) {
@@ -177,7 +177,7 @@ __global__ void __launch_bounds__(256) bias_rope_vnorm_kv_store_kernel(
     ss = wave_sum(ss);
     const float r = 1.0f / sqrtf(ss / (float)E + eps);
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < 8; ++u) {
       const int e = lane + 64 * u;
       if (e < E) dst[e] = Elem<T>::from_f(x[u] * r);
     }
@@ -261,7 +261,7 @@ __global__ void __launch_bounds__(256) local_attention_rows_kernel(LocalAttnArgs
   const T* vp = (const T*)a.v_pool;
   const bool sig = a.sigmoid != 0;
   const float hb = (sig && a.head_bias) ? a.head_bias[h] : 0.f;
-  float m = sig ? 0.f : -INFINITY, l = 0.f, acc[4] = {0.f, 0.f, 0.f, 0.f};
+  float m = sig ? 0.f : -INFINITY, l = 0.f, acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   constexpr int V = Elem<T>::kVec;
   // the kept first positions (none without a window), then the range that ends at the query
   for (int seg = n_first > 0 ? 0 : 1; seg < 2; ++seg) {
@@ -294,7 +294,7 @@ __global__ void __launch_bounds__(256) local_attention_rows_kernel(LocalAttnArgs
         p = valid ? expf(s - m_new) : 0.f;
         l = l * alpha + wave_sum(p);
 #pragma unroll
-        for (int u = 0; u < 4; ++u) acc[u] *= alpha;
+        for (int u = 0; u < 8; ++u) acc[u] *= alpha;
         m = m_new;
       }
       const int n = (int)((j_last - j0 + 1) < 64 ? (j_last - j0 + 1) : 64);
@@ -303,7 +303,7 @@ __global__ void __launch_bounds__(256) local_attention_rows_kernel(LocalAttnArgs
         const int sj = __shfl(slot, jj, 64);
         const T* v = vp + ((int64_t)sj * G + g) * E;
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < 8; ++u) {
           const int e = lane + 64 * u;
           if (e < E) acc[u] += pj * Elem<T>::to_f(v[e]);
         }
@@ -315,7 +315,7 @@ __global__ void __launch_bounds__(256) local_attention_rows_kernel(LocalAttnArgs
   T* o = (T*)a.out + t * a.out_ld + (int64_t)h * E;
   const T* gt = a.gate ? (const T*)a.gate + t * a.gate_ld + (int64_t)h * E : nullptr;
 #pragma unroll
-  for (int u = 0; u < 4; ++u) {
+  for (int u = 0; u < 8; ++u) {
     const int e = lane + 64 * u;
     if (e < E) {
       float y = acc[u] * inv;
@@ -880,8 +880,8 @@ static int launch_local_attention(LocalAttnArgs a, int64_t max_q_len, int form, 
   if (batch == 0 || num_tokens == 0) return 0;
   SEMIPD_CHECK_ARG(num_q_heads > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0, SEMIPD_ESHAPE,
                    "local_attention: %d query heads over %d key/value heads", num_q_heads, num_kv_heads);
-  SEMIPD_CHECK_ARG(qk_dim > 0 && qk_dim <= 512 && v_dim > 0 && v_dim <= 256, SEMIPD_ESHAPE,
-                   "local_attention: head sizes %d / %d (at most 512 / 256)", qk_dim, v_dim);
+  SEMIPD_CHECK_ARG(qk_dim > 0 && qk_dim <= 512 && v_dim > 0 && v_dim <= 512, SEMIPD_ESHAPE,
+                   "local_attention: head sizes %d / %d (at most 512 / 512)", qk_dim, v_dim);
   SEMIPD_CHECK_ARG(q && out && k_pool && v_pool && a.req_to_token && a.req_pool_indices && a.seq_lens, SEMIPD_EINVAL,
                    "local_attention: null pointer");
   SEMIPD_CHECK_ARG((q_start == nullptr) == (q_len == nullptr), SEMIPD_EINVAL, "local_attention: q_start and q_len come together");
@@ -967,8 +967,8 @@ extern "C" int semipd_bias_rope_vnorm_kv_store(void* qkv, int64_t ld, int64_t nu
                                                const void* bias_k, const void* bias_v, const int64_t* positions,
                                                const float* inv_freq, int rot_dims, float eps, void* k_pool, void* v_pool,
                                                const int64_t* loc, int dtype, void* stream) {
-  SEMIPD_CHECK_ARG(num_tokens >= 0 && num_q_heads > 0 && num_kv_heads > 0 && qk_dim > 0 && v_dim > 0 && v_dim <= 256, SEMIPD_EINVAL,
-                   "bias_rope_vnorm_kv_store: bad sizes (value rows of at most 256 elements)");
+  SEMIPD_CHECK_ARG(num_tokens >= 0 && num_q_heads > 0 && num_kv_heads > 0 && qk_dim > 0 && v_dim > 0 && v_dim <= 512, SEMIPD_EINVAL,
+                   "bias_rope_vnorm_kv_store: bad sizes (value rows of at most 512 elements)");
   SEMIPD_CHECK_ARG(rot_dims >= 0 && rot_dims <= qk_dim && rot_dims % 2 == 0, SEMIPD_EINVAL,
                    "bias_rope_vnorm_kv_store: %d rotated elements of a head of %d", rot_dims, qk_dim);
   if (num_tokens == 0) return 0;

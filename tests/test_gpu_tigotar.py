@@ -56,7 +56,7 @@ def test_dyn_tanh_seam(dtype, rows, width):
 
 # ----------------------------------------------------------------------------------------------- bias + rotation + value norm + store
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,G,D,E,rot", [(4, 2, 32, 16, 32), (3, 1, 20, 12, 10), (2, 2, 64, 256, 2), (1, 1, 128, 100, 0),
+@pytest.mark.parametrize("H,G,D,E,rot", [(4, 2, 32, 16, 32), (3, 1, 20, 12, 10), (2, 2, 64, 256, 2), (1, 1, 128, 100, 0), (2, 1, 8, 500, 4),
                                          (5, 5, 160, 8, 96)])
 def test_bias_rotation_value_norm_store(dtype, H, G, D, E, rot):
     from semi_pd_amd import ops
@@ -172,7 +172,7 @@ def test_window_attention_head_counts_and_sizes(H, G, D, E, dtype, form):
         torch.testing.assert_close(got, want, **_sum_tol(dtype, 54))
 
 
-@pytest.mark.parametrize("D,E", [(40, 24), (100, 7), (512, 8)])
+@pytest.mark.parametrize("D,E", [(40, 24), (100, 7), (512, 8), (32, 400)])
 def test_window_attention_sizes_only_the_row_form_takes(D, E):
     for dtype in (torch.bfloat16, torch.float32):
         got, want = _window_case(4, 2, D, E, 16, 3, dtype, 0, [(0, 35), (20, 1), (17, 9)], seed=D)
@@ -295,7 +295,7 @@ def test_min_gru_batches_of_unequal_requests(dtype):
 
 # ----------------------------------------------------------------------------------------------- experts
 @pytest.mark.parametrize("dtype,side_by_side", [(torch.float32, True), (torch.bfloat16, True), (torch.bfloat16, False)])
-@pytest.mark.parametrize("X,K,W,F,T", [(4, 2, 64, 32, 9), (6, 6, 128, 128, 70), (1, 1, 32, 16, 3), (3, 2, 100, 28, 17),
+@pytest.mark.parametrize("X,K,W,F,T", [(4, 2, 64, 32, 9), (6, 6, 128, 128, 70), (1, 1, 32, 16, 3), (3, 2, 100, 28, 17), (3, 2, 104, 30, 17),
                                        (8, 3, 256, 64, 700)])
 def test_ungated_experts(dtype, side_by_side, X, K, W, F, T, monkeypatch):
     from semi_pd_amd.layers.moe import UngatedMoE

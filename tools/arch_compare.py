@@ -1,4 +1,6 @@
-"""`python bench.py --arch-compare`: Kudirax next to the Llama-family model of equal size (random weights, one GPU).
+"""`python bench.py --arch-compare`: Kudirax next to the Llama-family model of equal size (random weights, one GPU);
+with `--arch-design tigotar`: Tigotar next to Kudirax, the closest model of the framework (fp32 stream, norms on the
+sublayers' outputs, attention over a bounded range of keys through the same kernel family), at equal layer sizes.
 
 Two parts, printed as one JSON object:
   * "models": prefill and decode throughput of a few-layer model of each design at layer sizes of real models, both driven
@@ -202,7 +204,161 @@ def _kernel_pairs(s, chunk, dev):
     return out
 
 
+TIGOTAR_SIZES = {
+    # experts x ff: `top` experts of ff = the dense feed-forward of the model next to it; the recurrence is as wide as the model
+    "8b-layer": dict(hidden=4096, heads=32, kv=8, dim=128, ff=14336, experts=8, top=2, layers=4, loop=(1, 3, 2), vocab=32000),
+    "3b-layer": dict(hidden=3072, heads=24, kv=8, dim=128, ff=8192, experts=8, top=2, layers=4, loop=(1, 3, 2), vocab=32000),
+    "1b-layer": dict(hidden=2048, heads=32, kv=8, dim=64, ff=8192, experts=16, top=4, layers=4, loop=(1, 3, 2), vocab=32000),
+}
+
+
+def _tigotar_kernel_pairs(s, window, keep, dev):
+    """[(what, Tigotar kernel's record, like kernel's record)] at the layer shape `s`."""
+    from semi_pd_amd import ops
+    from semi_pd_amd.layers.moe import fused_experts, fused_experts_ungated
+    dt = torch.bfloat16
+    H, G, D, W = s["heads"], s["kv"], s["dim"], s["hidden"]
+    X, K, F = s["experts"], s["top"], s["ff"] // s["top"]
+    E, R = D, W
+    out = []
+
+    def rec(t, nbytes=0.0, flops=0.0):
+        frac = max(nbytes / t / HBM, flops / t / MFMA)
+        return {"us": round(t * 1e6, 1), "TB_per_s": round(nbytes / t / 1e12, 2), "TFLOP_per_s": round(flops / t / 1e12, 1),
+                "of_roofline": round(frac, 3)}
+
+    # ---- prompt attention: 4 requests x 2048 new tokens; window of `window` + `keep` kept against blocks of `window` ----------
+    B, L = 4, 2048
+    T = B * L
+    kp = torch.randn(T + 1, G, D, device=dev, dtype=dt)
+    vp = torch.randn(T + 1, G, E, device=dev, dtype=dt)
+    r2t = (torch.arange(T, device=dev, dtype=torch.int32) + 1).view(B, L).contiguous()
+    q = torch.randn(T, H * D, device=dev, dtype=dt)
+    o = torch.empty(T, H * E, device=dev, dtype=dt)
+    hb = torch.full((H,), -3.0, device=dev)
+    sink = torch.zeros(H, device=dev)
+    rows = torch.arange(B, device=dev)
+    lens = torch.full((B,), L, device=dev, dtype=torch.int64)
+    q_start = (torch.arange(B, device=dev, dtype=torch.int32) * L)
+    q_len = torch.full((B,), L, device=dev, dtype=torch.int32)
+    t_new = _timed(lambda: ops.window_attention_fwd(q, o, kp, vp, r2t, rows, lens, q_start, q_len, L, D ** -0.5, window, keep, hb,
+                                                    True, None, 1.2))
+    pairs_new = B * sum(min(p + 1, window) + max(0, min(keep, p + 1 - window)) for p in range(L))
+    t_old = _timed(lambda: ops.local_attention_fwd(q, o, kp, vp, r2t, rows, lens, q_start, q_len, L, D ** -0.5, 30.0, window, sink, None))
+    pairs_old = B * sum((p % window) + 1 for p in range(L))
+    out.append((f"prompt attention, {B} x {L} tokens (window {window} + {keep} kept, sigmoid weights; like: blocks of {window}, softmax)",
+                rec(t_new, flops=2.0 * H * (D + E) * pairs_new), rec(t_old, flops=2.0 * H * (D + E) * pairs_old)))
+    # ---- decode attention: 32 requests at 2000 tokens ----------------------------------------------------------------
+    B2, C = 32, 2000
+    kp2 = torch.randn(B2 * C + 1, G, D, device=dev, dtype=dt)
+    vp2 = torch.randn(B2 * C + 1, G, E, device=dev, dtype=dt)
+    r2t2 = (torch.arange(B2 * C, device=dev, dtype=torch.int32) + 1).view(B2, C).contiguous()
+    q2 = torch.randn(B2, H * D, device=dev, dtype=dt)
+    o2 = torch.empty(B2, H * E, device=dev, dtype=dt)
+    rows2 = torch.arange(B2, device=dev)
+    lens2 = torch.full((B2,), C, device=dev, dtype=torch.int64)
+    t_new = _timed(lambda: ops.window_attention_fwd(q2, o2, kp2, vp2, r2t2, rows2, lens2, None, None, 1, D ** -0.5, window, keep, hb,
+                                                    True, None, 1.2))
+    keys_new = min(C, window) + max(0, min(keep, C - window))
+    t_old = _timed(lambda: ops.local_attention_fwd(q2, o2, kp2, vp2, r2t2, rows2, lens2, None, None, 1, D ** -0.5, 30.0, window, sink, None))
+    keys_old = ((C - 1) % window) + 1
+    out.append((f"decode attention, {B2} requests at {C} tokens ({keys_new} visible keys; like: {keys_old})",
+                rec(t_new, nbytes=B2 * G * (D + E) * 2.0 * keys_new), rec(t_old, nbytes=B2 * G * (D + E) * 2.0 * keys_old)))
+    # ---- the seam between two sublayers ----------------------------------------------------------------------------------
+    for Tn in (8192, 32):
+        y = torch.randn(Tn, W, device=dev, dtype=dt)
+        res = torch.randn(Tn, W, device=dev, dtype=torch.float32)
+        w = torch.ones(W, device=dev, dtype=dt)
+        b = torch.zeros(W, device=dev, dtype=dt)
+        al = torch.tensor(0.5, device=dev, dtype=dt)
+        t_new = _timed(lambda: ops.dyn_tanh(y, (w, b, al), residual=res, params_out=(w, b, al)))
+        t_old = _timed(lambda: ops.layernorm(y, w, b, 1e-5, residual=res, in_bias=b))
+        nb = Tn * W * (2 + 4 + 4 + 2.0)
+        out.append((f"stream += squash(y), next input = squash(stream), {Tn} rows of {W} (like: LayerNorm + residual add)",
+                    rec(t_new, nbytes=nb), rec(t_old, nbytes=nb)))
+    # ---- the step between the projection and the attention ---------------------------------------------------------------
+    Tn = 8192
+    cols = H * D + G * D + G * E + 3 * R
+    p = torch.randn(Tn, cols, device=dev, dtype=dt)
+    kp3 = torch.zeros(Tn + 1, G, D, device=dev, dtype=dt)
+    vp3 = torch.zeros(Tn + 1, G, E, device=dev, dtype=dt)
+    loc = torch.arange(1, Tn + 1, device=dev)
+    pos = torch.arange(Tn, device=dev)
+    bq, bk, bv = (torch.zeros(n, device=dev, dtype=dt) for n in (H * D, G * D, G * E))
+    inv_freq = 10000.0 ** (-2.0 * torch.arange(D // 2, dtype=torch.float32, device=dev) / D)
+    t_new = _timed(lambda: ops.bias_rope_vnorm_kv_store(p, H, G, D, E, H * D, H * D + G * D, bq, bk, bv, pos, inv_freq, D, 1e-6, kp3, vp3, loc))
+    pk = torch.randn(Tn, H * D + G * D + G * E + H * E, device=dev, dtype=dt)
+    t_old = _timed(lambda: ops.unit_norm_and_store_kv(pk, H, G, D, E, H * D, H * D + G * D, 1e-5, kp3, vp3, loc))
+    nb = Tn * 2.0 * (2 * H * D + 2 * G * D + 2 * G * E)
+    out.append((f"q / k / v preparation + KV-pool store, {Tn} tokens (biases, pair rotation, value norm; like: unit norm of q and k)",
+                rec(t_new, nbytes=nb), rec(t_old, nbytes=nb)))
+    # ---- the recurrence: a prompt batch (chunked form) and a decode batch ---------------------------------------------------
+    state = torch.zeros(B2 + 1, R, device=dev)
+    yb = torch.empty(Tn, R, device=dev, dtype=dt)
+    u = torch.randn(Tn, R, device=dev, dtype=dt)
+    bb = torch.zeros(R, device=dev, dtype=dt)
+    st4 = torch.arange(1, B + 1, device=dev)
+    t_new = _timed(lambda: ops.min_gru(p, H * D + G * D + G * E, H * D + G * D + G * E + R, H * D + G * D + G * E + 2 * R, R, bb, bb, yb,
+                                       state, st4, lens, q_start, q_len, L))
+    t_old = _timed(lambda: ops.bias_relu_square_(u, bb))
+    out.append((f"minGRU over {B} x {L} tokens, {R} channels (three passes over chunks of 64; like: an in-place element-wise kernel over as many rows)",
+                rec(t_new, nbytes=Tn * R * 2.0 * (3 + 2 + 1)), rec(t_old, nbytes=Tn * R * 2.0 * 2)))
+    pd = torch.randn(B2, cols, device=dev, dtype=dt)
+    yd = torch.empty(B2, R, device=dev, dtype=dt)
+    ud = torch.randn(B2, R, device=dev, dtype=dt)
+    st32 = torch.arange(1, B2 + 1, device=dev)
+    t_new = _timed(lambda: ops.min_gru(pd, H * D + G * D + G * E, H * D + G * D + G * E + R, H * D + G * D + G * E + 2 * R, R, bb, bb, yd,
+                                       state, st32, lens2, None, None, 1))
+    t_old = _timed(lambda: ops.bias_relu_square_(ud, bb))
+    out.append((f"minGRU decode step, {B2} requests, {R} channels (like: an in-place element-wise kernel over as many rows; both are launch-bound)",
+                rec(t_new, nbytes=B2 * R * (2.0 * 4 + 8)), rec(t_old, nbytes=B2 * R * 2.0 * 2)))
+    # ---- experts: ungated (two GEMMs per expert) against gated SiLU (three), same sizes ----------------------------------------
+    w_up = torch.randn(X, F, W, device=dev, dtype=dt) * 0.02
+    w_down = torch.randn(X, W, F, device=dev, dtype=dt) * 0.02
+    w13 = torch.randn(X, 2 * F, W, device=dev, dtype=dt) * 0.02
+    for Tn in (8192, 32):
+        h = torch.randn(Tn, W, device=dev, dtype=dt)
+        tw, ti = ops.topk_softmax(torch.randn(Tn, X, device=dev), K, True)
+        t_new = _timed(lambda: fused_experts_ungated(h, w_up, w_down, tw, ti))
+        t_old = _timed(lambda: fused_experts(h, w13, w_down, tw, ti))
+        if Tn > 1024:
+            new, old = rec(t_new, flops=2.0 * Tn * K * 2 * W * F), rec(t_old, flops=2.0 * Tn * K * 3 * W * F)
+        else:   # every expert is touched: the call streams all weights once
+            new, old = rec(t_new, nbytes=X * 2.0 * W * F * 2), rec(t_old, nbytes=X * 3.0 * W * F * 2)
+        out.append((f"experts, {Tn} tokens, top {K} of {X} x {F} (up, squared ReLU, down; like: gate | up, SiLU * mul, down)", new, old))
+    return out
+
+
+def main_tigotar(args) -> dict:
+    from semi_pd_amd.models.kudirax import kudirax_uniform
+    from semi_pd_amd.models.tigotar import tigotar_uniform
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    window, keep = int(getattr(args, "arch_chunk", 1024) or 1024), 4
+    names = [n for n in (getattr(args, "arch_sizes", "") or ",".join(TIGOTAR_SIZES)).split(",") if n]
+    result = {"what": "Tigotar next to Kudirax at equal layer sizes", "dtype": "bf16", "data": "synthetic", "window": window,
+              "kept_first": keep, "models": {}, "kernels": {}}
+    for name in names:
+        s = TIGOTAR_SIZES[name]
+        result["kernels"][name] = [
+            {"kernel": what, "tigotar": new, "like": old,
+             "roofline_fraction_ratio": round(new["of_roofline"] / max(old["of_roofline"], 1e-9), 2)}
+            for what, new, old in _tigotar_kernel_pairs(s, window, keep, dev)]
+        tcfg = tigotar_uniform(s["vocab"], s["hidden"], s["layers"], s["heads"], s["kv"], s["dim"], s["dim"], s["hidden"],
+                               s["experts"], s["top"], s["ff"] // s["top"], window, keep, loop=s["loop"])
+        runs = len(tcfg.runs())
+        kcfg = kudirax_uniform(s["vocab"], s["hidden"], runs, s["heads"], s["kv"], s["dim"], s["dim"], s["ff"], window)
+        result["models"][name] = {
+            "layer_runs": runs,
+            "tigotar": _model_throughput(tcfg, 2048, 4, 32, 1100, 20),
+            "kudirax": _model_throughput(kcfg, 2048, 4, 32, 1100, 20)}
+    print(json.dumps(result), flush=True)
+    return result
+
+
 def main(args) -> dict:
+    if getattr(args, "arch_design", "kudirax") == "tigotar":
+        return main_tigotar(args)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     chunk = int(getattr(args, "arch_chunk", 1024) or 0)
