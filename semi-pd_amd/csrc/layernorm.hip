@@ -136,36 +136,36 @@ __global__ void __launch_bounds__(256) layernorm_vec_kernel(const TIn* __restric
   }
 }
 
-// 8 elements per thread and step, 16-byte accesses (width % 8 == 0, rows 16-byte aligned)
+// 8 elements per thread and step, 16-byte accesses (width % 8 == 0, rows 16-byte aligned); a workgroup walks whole rows
 template <typename T>
 __global__ void __launch_bounds__(256) bias_relu_square_vec_kernel(T* __restrict__ u, int64_t ld, const T* __restrict__ bias,
                                                                    int64_t rows, int64_t width) {
-  const int64_t per_row = width >> 3, n = rows * per_row;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
-    const int64_t r = i / per_row, c = (i - r * per_row) << 3;
-    T* p = u + r * ld + c;
-    float v[8];
-    if constexpr (sizeof(T) == 2) {
-      const Vec16<T> a = load16(p);
+  for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
+    for (int64_t c = (int64_t)threadIdx.x * 8; c < width; c += (int64_t)blockDim.x * 8) {
+      T* p = u + r * ld + c;
+      float v[8];
+      if constexpr (sizeof(T) == 2) {
+        const Vec16<T> a = load16(p);
 #pragma unroll
-      for (int k = 0; k < 8; ++k) v[k] = Elem<T>::to_f(a.e[k]);
-    } else {
+        for (int k = 0; k < 8; ++k) v[k] = Elem<T>::to_f(a.e[k]);
+      } else {
 #pragma unroll
-      for (int k = 0; k < 8; ++k) v[k] = Elem<T>::to_f(p[k]);
-    }
+        for (int k = 0; k < 8; ++k) v[k] = Elem<T>::to_f(p[k]);
+      }
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      if (bias) v[k] += Elem<T>::to_f(bias[c + k]);
-      v[k] = v[k] > 0.f ? v[k] * v[k] : 0.f;
-    }
-    if constexpr (sizeof(T) == 2) {
-      Vec16<T> o;
+      for (int k = 0; k < 8; ++k) {
+        if (bias) v[k] += Elem<T>::to_f(bias[c + k]);
+        v[k] = v[k] > 0.f ? v[k] * v[k] : 0.f;
+      }
+      if constexpr (sizeof(T) == 2) {
+        Vec16<T> o;
 #pragma unroll
-      for (int k = 0; k < 8; ++k) o.e[k] = Elem<T>::from_f(v[k]);
-      store16(p, o);
-    } else {
+        for (int k = 0; k < 8; ++k) o.e[k] = Elem<T>::from_f(v[k]);
+        store16(p, o);
+      } else {
 #pragma unroll
-      for (int k = 0; k < 8; ++k) p[k] = Elem<T>::from_f(v[k]);
+        for (int k = 0; k < 8; ++k) p[k] = Elem<T>::from_f(v[k]);
+      }
     }
   }
 }
@@ -185,7 +185,20 @@ __global__ void __launch_bounds__(256) bias_relu_square_kernel(T* __restrict__ u
 
 
 // ------------------------------------------------------------------------------------------------ dynamic tanh
-// V elements per thread (V = 8: 16-byte accesses on 16-bit rows; V = 1: any width and alignment)
+// tanh in fp32 from one v_exp_f32 and one v_rcp_f32: 1 - 2 / (exp(2 |a|) + 1) with the sign put back (overflow of the
+// exponential gives 1); below |a| = 0.04, where that difference cancels, the odd series a (1 - a^2 / 3 + 2 a^4 / 15)
+// (its next term is below 1e-10 relative there).  Within a few ulp of tanhf at a fraction of its instructions: the kernel
+// has two of them per element and is otherwise bound by memory.
+__device__ __forceinline__ float tanh_fast(float a) {
+  const float x = fabsf(a);
+  const float e = __builtin_amdgcn_exp2f(x * 2.8853900817779268f);          // exp(2 x)
+  const float big = 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+  const float a2 = a * a;
+  const float small = x * (1.0f + a2 * (-0.33333333333f + a2 * 0.13333333333f));
+  return copysignf(x < 0.04f ? small : big, a);
+}
+
+// A workgroup per row; V elements per thread and step (V = 8: 16-byte accesses on 16-bit rows; V = 1: any width and alignment)
 template <typename T, typename TIn, int V>
 __global__ void __launch_bounds__(256) dyn_tanh_kernel(const TIn* __restrict__ y, int64_t y_ld, const T* __restrict__ wa,
                                                        const T* __restrict__ ba, const T* __restrict__ alpha_a,
@@ -193,50 +206,75 @@ __global__ void __launch_bounds__(256) dyn_tanh_kernel(const TIn* __restrict__ y
                                                        const T* __restrict__ wb, const T* __restrict__ bb,
                                                        const T* __restrict__ alpha_b, T* __restrict__ out, int64_t out_ld,
                                                        int64_t rows, int64_t width) {
-  const int64_t per_row = width / V, n = rows * per_row;
   const float aa = alpha_a ? Elem<T>::to_f(alpha_a[0]) : 0.f, ab = alpha_b ? Elem<T>::to_f(alpha_b[0]) : 0.f;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
-    const int64_t r = i / per_row, c = (i - r * per_row) * V;
-    float v[V];
+  for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
+    for (int64_t c = (int64_t)threadIdx.x * V; c < width; c += (int64_t)blockDim.x * V) {
+      float v[V];
 #pragma unroll
-    for (int k = 0; k < V; ++k) v[k] = 0.f;
-    if (y) {
-      if constexpr (V == 8 && sizeof(TIn) == 2) {
-        const Vec16<TIn> a = load16(y + r * y_ld + c);
-#pragma unroll
-        for (int k = 0; k < V; ++k) v[k] = Elem<TIn>::to_f(a.e[k]);
-      } else {
-#pragma unroll
-        for (int k = 0; k < V; ++k) v[k] = Elem<TIn>::to_f(y[r * y_ld + c + k]);
-      }
-#pragma unroll
-      for (int k = 0; k < V; ++k) v[k] = tanhf(aa * v[k]) * Elem<T>::to_f(wa[c + k]) + Elem<T>::to_f(ba[c + k]);
-    }
-    if (residual) {
-      float* rp = residual + r * res_ld + c;
-      if (accumulate || !y) {
-#pragma unroll
-        for (int k = 0; k < V; ++k) v[k] += rp[k];
-      }
+      for (int k = 0; k < V; ++k) v[k] = 0.f;
       if (y) {
+        float w[V], b[V];
+        if constexpr (V == 8 && sizeof(TIn) == 2) {
+          const Vec16<TIn> a = load16(y + r * y_ld + c);
 #pragma unroll
-        for (int k = 0; k < V; ++k) rp[k] = v[k];
+          for (int k = 0; k < V; ++k) v[k] = Elem<TIn>::to_f(a.e[k]);
+        } else {
+#pragma unroll
+          for (int k = 0; k < V; ++k) v[k] = Elem<TIn>::to_f(y[r * y_ld + c + k]);
+        }
+        if constexpr (V == 8 && sizeof(T) == 2) {
+          const Vec16<T> w8 = load16(wa + c), b8 = load16(ba + c);
+#pragma unroll
+          for (int k = 0; k < V; ++k) {
+            w[k] = Elem<T>::to_f(w8.e[k]);
+            b[k] = Elem<T>::to_f(b8.e[k]);
+          }
+        } else {
+#pragma unroll
+          for (int k = 0; k < V; ++k) {
+            w[k] = Elem<T>::to_f(wa[c + k]);
+            b[k] = Elem<T>::to_f(ba[c + k]);
+          }
+        }
+#pragma unroll
+        for (int k = 0; k < V; ++k) v[k] = tanh_fast(aa * v[k]) * w[k] + b[k];
       }
-    }
-    if (out) {
-      if (wb) {
+      if (residual) {
+        float* rp = residual + r * res_ld + c;
+        if (accumulate || !y) {
+          if constexpr (V == 8) {
+            const float4 a = *reinterpret_cast<const float4*>(rp), d = *reinterpret_cast<const float4*>(rp + 4);
+            v[0] += a.x; v[1] += a.y; v[2] += a.z; v[3] += a.w; v[4] += d.x; v[5] += d.y; v[6] += d.z; v[7] += d.w;
+          } else {
 #pragma unroll
-        for (int k = 0; k < V; ++k) v[k] = tanhf(ab * v[k]) * Elem<T>::to_f(wb[c + k]) + Elem<T>::to_f(bb[c + k]);
+            for (int k = 0; k < V; ++k) v[k] += rp[k];
+          }
+        }
+        if (y) {
+          if constexpr (V == 8) {
+            *reinterpret_cast<float4*>(rp) = float4{v[0], v[1], v[2], v[3]};
+            *reinterpret_cast<float4*>(rp + 4) = float4{v[4], v[5], v[6], v[7]};
+          } else {
+#pragma unroll
+            for (int k = 0; k < V; ++k) rp[k] = v[k];
+          }
+        }
       }
-      T* op = out + r * out_ld + c;
-      if constexpr (V == 8 && sizeof(T) == 2) {
-        Vec16<T> o;
+      if (out) {
+        if (wb) {
 #pragma unroll
-        for (int k = 0; k < V; ++k) o.e[k] = Elem<T>::from_f(v[k]);
-        store16(op, o);
-      } else {
+          for (int k = 0; k < V; ++k) v[k] = tanh_fast(ab * v[k]) * Elem<T>::to_f(wb[c + k]) + Elem<T>::to_f(bb[c + k]);
+        }
+        T* op = out + r * out_ld + c;
+        if constexpr (V == 8 && sizeof(T) == 2) {
+          Vec16<T> o;
 #pragma unroll
-        for (int k = 0; k < V; ++k) op[k] = Elem<T>::from_f(v[k]);
+          for (int k = 0; k < V; ++k) o.e[k] = Elem<T>::from_f(v[k]);
+          store16(op, o);
+        } else {
+#pragma unroll
+          for (int k = 0; k < V; ++k) op[k] = Elem<T>::from_f(v[k]);
+        }
       }
     }
   }
@@ -316,10 +354,10 @@ extern "C" int semipd_bias_relu_square(void* u, int64_t ld, const void* bias, in
   const int64_t n = rows * width;
   const int64_t esz = dtype == SEMIPD_F32 ? 4 : 2;
   if (width % 8 == 0 && aligned16(u) && (ld * esz) % 16 == 0) {
-    const int64_t nv = n / 8;
-    const unsigned vblocks = (unsigned)((nv + 255) / 256 < 16384 ? (nv + 255) / 256 : 16384);
+    const unsigned vblocks = (unsigned)(rows < (1 << 20) ? rows : (1 << 20));
+    const unsigned threads = (unsigned)(width / 8 >= 256 ? 256 : (width / 8 + 63) / 64 * 64);
     SEMIPD_DISPATCH_DTYPE(dtype, T,
-                          hipLaunchKernelGGL((bias_relu_square_vec_kernel<T>), dim3(vblocks), dim3(256), 0, as_stream(stream),
+                          hipLaunchKernelGGL((bias_relu_square_vec_kernel<T>), dim3(vblocks), dim3(threads), 0, as_stream(stream),
                                              (T*)u, ld, (const T*)bias, rows, width));
     return launch_status("bias_relu_square");
   }
@@ -342,12 +380,14 @@ extern "C" int semipd_dyn_tanh(const void* in, int64_t in_ld, int in_is_f32, con
                    "dyn_tanh: the output's weight, bias and alpha come together");
   SEMIPD_CHECK_ARG(!weight_b || out, SEMIPD_EINVAL, "dyn_tanh: output parameters without an output");
   const int64_t esz = dtype == SEMIPD_F32 ? 4 : 2, in_esz = in_is_f32 ? 4 : esz;
-  const bool vec = width % 8 == 0 && (!in || (aligned16(in) && (in_ld * in_esz) % 16 == 0)) &&
+  const bool vec = width % 8 == 0 && (!in || (aligned16(in) && (in_ld * in_esz) % 16 == 0 && aligned16(weight_a) && aligned16(bias_a))) &&
                    (!residual || (aligned16(residual) && residual_ld % 4 == 0)) && (!out || (aligned16(out) && (out_ld * esz) % 16 == 0));
-  const int64_t n = rows * width / (vec ? 8 : 1);
-  const unsigned blocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
+  const unsigned blocks = (unsigned)(rows < (1 << 20) ? rows : (1 << 20));
+  // (narrow rows: as many waves as the row has work for)
+  const int64_t per_row = (width + (vec ? 8 : 1) - 1) / (vec ? 8 : 1);
+  const unsigned threads = (unsigned)(per_row >= 256 ? 256 : (per_row + 63) / 64 * 64);
 #define SEMIPD_DYT(TIN, VV)                                                                                                     \
-  hipLaunchKernelGGL((dyn_tanh_kernel<T, TIN, VV>), dim3(blocks), dim3(256), 0, as_stream(stream), (const TIN*)in, in_ld,          \
+  hipLaunchKernelGGL((dyn_tanh_kernel<T, TIN, VV>), dim3(blocks), dim3(threads), 0, as_stream(stream), (const TIN*)in, in_ld,          \
                      (const T*)weight_a, (const T*)bias_a, (const T*)alpha_a, residual, residual_ld, accumulate,                 \
                      (const T*)weight_b, (const T*)bias_b, (const T*)alpha_b, (T*)out, out_ld, rows, width)
   SEMIPD_DISPATCH_DTYPE(dtype, T, {

@@ -184,6 +184,97 @@ __global__ void __launch_bounds__(256) bias_rope_vnorm_kv_store_kernel(
   }
 }
 
+// The same for 16-bit types with 16-byte accesses, one wave per TOKEN: the cosines and sines of the token's angles are
+// computed once (into LDS) and serve every q and k head; a head of q / k is D / 8 pieces of four pairs, taken by the lanes in
+// turn; value heads go Lp lanes each (the power of two above E / 8) with the sum of squares reduced inside the group.
+// D, E, rot multiples of 8 (a piece is rotated wholly or not at all), rot <= 512, E <= 512.
+template <typename T>
+__global__ void __launch_bounds__(256) bias_rope_vnorm_kv_store_vec_kernel(
+    T* __restrict__ qkv, int64_t ld, int64_t num_tokens, int H, int G, int D, int E, int64_t k_off, int64_t v_off,
+    const T* __restrict__ bq, const T* __restrict__ bk, const T* __restrict__ bv, const int64_t* __restrict__ positions,
+    const float* __restrict__ inv_freq, int rot, float eps, T* __restrict__ k_pool, T* __restrict__ v_pool,
+    const int64_t* __restrict__ loc) {
+  __shared__ float cs_lds[4][2][256];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t t = (int64_t)blockIdx.x * 4 + wave;
+  if (t >= num_tokens) return;            // (whole waves leave: what follows synchronises inside a wave only)
+  const float pos = (float)positions[t];
+  for (int i = lane; i < rot / 2; i += 64) {
+    float sn, cs;
+    sincosf(pos * inv_freq[i], &sn, &cs);
+    cs_lds[wave][0][i] = cs;
+    cs_lds[wave][1][i] = sn;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  T* row = qkv + t * ld;
+  const int64_t slot = loc[t];
+  const int L = D >> 3, n_qk = (H + G) * L;
+  for (int idx = lane; idx < n_qk; idx += 64) {
+    const int h = idx / L, pc = idx - h * L;
+    const bool is_q = h < H;
+    const int hh = is_q ? h : h - H;
+    T* src = (is_q ? row + (int64_t)h * D : row + k_off + (int64_t)hh * D) + pc * 8;
+    const Vec16<T> x = load16(src);
+    float f[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) f[u] = Elem<T>::to_f(x.e[u]);
+    const T* bias = is_q ? bq : bk;
+    if (bias) {
+      const Vec16<T> bb = load16(bias + hh * D + pc * 8);
+#pragma unroll
+      for (int u = 0; u < 8; ++u) f[u] += Elem<T>::to_f(bb.e[u]);
+    }
+    if (pc * 8 < rot) {
+      const float4 c4 = *reinterpret_cast<const float4*>(&cs_lds[wave][0][pc * 4]);
+      const float4 s4 = *reinterpret_cast<const float4*>(&cs_lds[wave][1][pc * 4]);
+      const float cs[4] = {c4.x, c4.y, c4.z, c4.w}, sn[4] = {s4.x, s4.y, s4.z, s4.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float x0 = f[2 * j], x1 = f[2 * j + 1];
+        f[2 * j] = x0 * cs[j] - x1 * sn[j];
+        f[2 * j + 1] = x1 * cs[j] + x0 * sn[j];
+      }
+    }
+    Vec16<T> y;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) y.e[u] = Elem<T>::from_f(f[u]);
+    store16(is_q ? src : k_pool + (slot * G + hh) * D + pc * 8, y);
+  }
+  const int LV = E >> 3;
+  int Lp = 1;
+  while (Lp < LV) Lp <<= 1;
+  const int per_iter = 64 / Lp, sl = lane & (Lp - 1);
+  for (int g0 = 0; g0 < G; g0 += per_iter) {
+    const int g = g0 + lane / Lp;
+    const bool on = g < G && sl < LV;
+    float f[8], ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) f[u] = 0.f;
+    if (on) {
+      const Vec16<T> x = load16(row + v_off + (int64_t)g * E + sl * 8);
+#pragma unroll
+      for (int u = 0; u < 8; ++u) f[u] = Elem<T>::to_f(x.e[u]);
+      if (bv) {
+        const Vec16<T> bb = load16(bv + g * E + sl * 8);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) f[u] += Elem<T>::to_f(bb.e[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) ss += f[u] * f[u];
+    }
+    for (int o = Lp >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+    if (on) {
+      const float r = 1.0f / sqrtf(ss / (float)E + eps);
+      Vec16<T> y;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) y.e[u] = Elem<T>::from_f(f[u] * r);
+      store16(v_pool + (slot * G + g) * E + sl * 8, y);
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ shared pieces
 struct LocalAttnArgs {
   const void* q; int64_t q_ld;
@@ -977,6 +1068,17 @@ extern "C" int semipd_bias_rope_vnorm_kv_store(void* qkv, int64_t ld, int64_t nu
   SEMIPD_CHECK_ARG(ld >= v_off + (int64_t)num_kv_heads * v_dim && k_off >= (int64_t)num_q_heads * qk_dim &&
                        v_off >= k_off + (int64_t)num_kv_heads * qk_dim,
                    SEMIPD_EINVAL, "bias_rope_vnorm_kv_store: column ranges overlap or leave the row");
+  if ((dtype == SEMIPD_BF16 || dtype == SEMIPD_F16) && qk_dim % 8 == 0 && v_dim % 8 == 0 && rot_dims % 8 == 0 && rot_dims <= 512 &&
+      ld % 8 == 0 && k_off % 8 == 0 && v_off % 8 == 0 && aligned16(qkv) && aligned16(k_pool) && aligned16(v_pool) &&
+      (!bias_q || aligned16(bias_q)) && (!bias_k || aligned16(bias_k)) && (!bias_v || aligned16(bias_v))) {
+    const unsigned vb = (unsigned)((num_tokens + 3) / 4);
+    SEMIPD_DISPATCH_HALF(dtype, T,
+                         hipLaunchKernelGGL((bias_rope_vnorm_kv_store_vec_kernel<T>), dim3(vb), dim3(256), 0, as_stream(stream),
+                                            (T*)qkv, ld, num_tokens, num_q_heads, num_kv_heads, qk_dim, v_dim, k_off, v_off,
+                                            (const T*)bias_q, (const T*)bias_k, (const T*)bias_v, positions, inv_freq, rot_dims,
+                                            eps, (T*)k_pool, (T*)v_pool, loc));
+    return launch_status("bias_rope_vnorm_kv_store");
+  }
   const int64_t items = num_tokens * (num_q_heads + 2 * num_kv_heads);
   const unsigned blocks = (unsigned)((items + 3) / 4);
   SEMIPD_DISPATCH_DTYPE(dtype, T,

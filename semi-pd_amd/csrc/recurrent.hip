@@ -37,35 +37,99 @@ struct MinGruArgs {
 
 constexpr int kChunk = 64;
 
-__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
-
-template <typename T>
-__device__ __forceinline__ void gru_step(const T* row, const MinGruArgs& a, int c, float bz, float bx, float& S, float& keep) {
-  const float z = sigmoidf_(Elem<T>::to_f(row[a.z_off + c]) + bz);
-  const float u = Elem<T>::to_f(row[a.x_off + c]) + bx;
-  const float cand = u >= 0.f ? u + 0.5f : sigmoidf_(u);
-  keep = 1.0f - z;
-  S = keep * S + z * cand;
+// 1 / (1 + exp(-x)) from one v_exp_f32 and one v_rcp_f32 (overflow of the exponential gives 0)
+__device__ __forceinline__ float sigmoidf_(float x) {
+  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
 }
 
-template <typename T>
+// V adjacent channels of one row as floats (V = 4: one 8- or 16-byte access)
+template <typename T, int V> __device__ __forceinline__ void load_ch(const T* p, float (&f)[V]) {
+  if constexpr (V == 4 && sizeof(T) == 2) {
+    const uint2 w = *reinterpret_cast<const uint2*>(p);
+    T e[4];
+    __builtin_memcpy(e, &w, 8);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) f[k] = Elem<T>::to_f(e[k]);
+  } else if constexpr (V == 4) {
+    const float4 w = *reinterpret_cast<const float4*>(p);
+    f[0] = w.x; f[1] = w.y; f[2] = w.z; f[3] = w.w;
+  } else {
+#pragma unroll
+    for (int k = 0; k < V; ++k) f[k] = Elem<T>::to_f(p[k]);
+  }
+}
+template <typename T, int V> __device__ __forceinline__ void store_ch(T* p, const float (&f)[V]) {
+  if constexpr (V == 4 && sizeof(T) == 2) {
+    T e[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) e[k] = Elem<T>::from_f(f[k]);
+    uint2 w;
+    __builtin_memcpy(&w, e, 8);
+    *reinterpret_cast<uint2*>(p) = w;
+  } else if constexpr (V == 4) {
+    *reinterpret_cast<float4*>(p) = float4{f[0], f[1], f[2], f[3]};
+  } else {
+#pragma unroll
+    for (int k = 0; k < V; ++k) p[k] = Elem<T>::from_f(f[k]);
+  }
+}
+
+// one row of V channels: S <- (1 - z) S + z cand; keep = 1 - z
+template <typename T, int V>
+__device__ __forceinline__ void gru_step(const T* row, const MinGruArgs& a, int c, const float (&bz)[V], const float (&bx)[V],
+                                         float (&S)[V], float (&keep)[V]) {
+  float zl[V], xl[V];
+  load_ch<T, V>(row + a.z_off + c, zl);
+  load_ch<T, V>(row + a.x_off + c, xl);
+#pragma unroll
+  for (int k = 0; k < V; ++k) {
+    const float z = sigmoidf_(zl[k] + bz[k]);
+    const float u = xl[k] + bx[k];
+    const float cand = u >= 0.f ? u + 0.5f : sigmoidf_(u);
+    keep[k] = 1.0f - z;
+    S[k] = keep[k] * S[k] + z * cand;
+  }
+}
+
+template <typename T, int V>
+__device__ __forceinline__ void gru_out(const T* row, const MinGruArgs& a, int c, const float (&S)[V], T* y) {
+  float g[V], o[V];
+  load_ch<T, V>(row + a.g_off + c, g);
+#pragma unroll
+  for (int k = 0; k < V; ++k) o[k] = a.out_scale * S[k] * (g[k] * sigmoidf_(g[k]));
+  store_ch<T, V>(y + c, o);
+}
+
+template <typename T, int V>
+__device__ __forceinline__ void load_biases(const MinGruArgs& a, int c, float (&bz)[V], float (&bx)[V]) {
+#pragma unroll
+  for (int k = 0; k < V; ++k) {
+    bz[k] = a.bz ? Elem<T>::to_f(((const T*)a.bz)[c + k]) : 0.f;
+    bx[k] = a.bx ? Elem<T>::to_f(((const T*)a.bx)[c + k]) : 0.f;
+  }
+}
+
+template <typename T, int V>
 __global__ void __launch_bounds__(256) min_gru_rows_kernel(MinGruArgs a) {
-  const int c = blockIdx.x * 256 + threadIdx.x;
+  const int c = (blockIdx.x * 256 + threadIdx.x) * V;
   const int b = blockIdx.y;
   if (c >= a.R) return;
   const int64_t n = a.q_len ? a.q_len[b] : 1, t0 = a.q_start ? a.q_start[b] : b;
   if (n <= 0) return;
   const int64_t first_pos = a.seq_lens[b] - n;
   float* sp = a.state + a.state_indices[b] * a.state_ld + c;
-  float S = first_pos > 0 ? *sp : 0.f, keep;
-  const float bz = a.bz ? Elem<T>::to_f(((const T*)a.bz)[c]) : 0.f, bx = a.bx ? Elem<T>::to_f(((const T*)a.bx)[c]) : 0.f;
+  float S[V], keep[V], bz[V], bx[V];
+#pragma unroll
+  for (int k = 0; k < V; ++k) S[k] = first_pos > 0 ? sp[k] : 0.f;
+  load_biases<T, V>(a, c, bz, bx);
+#pragma unroll 2
   for (int64_t i = 0; i < n; ++i) {
     const T* row = (const T*)a.p + (t0 + i) * a.ld;
-    gru_step<T>(row, a, c, bz, bx, S, keep);
-    const float g = Elem<T>::to_f(row[a.g_off + c]);
-    ((T*)a.y)[(t0 + i) * a.y_ld + c] = Elem<T>::from_f(a.out_scale * S * (g * sigmoidf_(g)));
+    gru_step<T, V>(row, a, c, bz, bx, S, keep);
+    gru_out<T, V>(row, a, c, S, (T*)a.y + (t0 + i) * a.y_ld);
   }
-  *sp = S;
+#pragma unroll
+  for (int k = 0; k < V; ++k) sp[k] = S[k];
 }
 
 // which request and which of its chunks chunk id `id` is (chunks are counted request after request)
@@ -83,29 +147,38 @@ __device__ __forceinline__ bool locate_chunk(const MinGruArgs& a, int64_t id, in
   return false;
 }
 
-template <typename T, bool WRITE>
+template <typename T, int V, bool WRITE>
 __global__ void __launch_bounds__(256) min_gru_chunk_kernel(MinGruArgs a) {
-  const int c = blockIdx.x * 256 + threadIdx.x;
+  const int c = (blockIdx.x * 256 + threadIdx.x) * V;
   int b;
   int64_t k;
   if (c >= a.R || !locate_chunk(a, blockIdx.y, b, k)) return;
   const int64_t n = a.q_len[b], i0 = k * kChunk, i1 = i0 + kChunk < n ? i0 + kChunk : n, t0 = a.q_start[b];
-  const float bz = a.bz ? Elem<T>::to_f(((const T*)a.bz)[c]) : 0.f, bx = a.bx ? Elem<T>::to_f(((const T*)a.bx)[c]) : 0.f;
+  float S[V], A[V], keep[V], bz[V], bx[V];
+  load_biases<T, V>(a, c, bz, bx);
   float* wk = a.work + (int64_t)blockIdx.y * 2 * a.R;
-  float S = WRITE ? wk[a.R + c] : 0.f, A = 1.0f, keep;
+#pragma unroll
+  for (int j = 0; j < V; ++j) {
+    S[j] = WRITE ? wk[a.R + c + j] : 0.f;
+    A[j] = 1.0f;
+  }
+#pragma unroll 4
   for (int64_t i = i0; i < i1; ++i) {
     const T* row = (const T*)a.p + (t0 + i) * a.ld;
-    gru_step<T>(row, a, c, bz, bx, S, keep);
+    gru_step<T, V>(row, a, c, bz, bx, S, keep);
     if constexpr (WRITE) {
-      const float g = Elem<T>::to_f(row[a.g_off + c]);
-      ((T*)a.y)[(t0 + i) * a.y_ld + c] = Elem<T>::from_f(a.out_scale * S * (g * sigmoidf_(g)));
+      gru_out<T, V>(row, a, c, S, (T*)a.y + (t0 + i) * a.y_ld);
     } else {
-      A *= keep;
+#pragma unroll
+      for (int j = 0; j < V; ++j) A[j] *= keep[j];
     }
   }
   if constexpr (!WRITE) {
-    wk[c] = A;
-    wk[a.R + c] = S;
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      wk[c + j] = A[j];
+      wk[a.R + c + j] = S[j];
+    }
   }
 }
 
@@ -154,21 +227,31 @@ extern "C" int semipd_min_gru(const void* proj, int64_t ld, int64_t z_off, int64
   SEMIPD_CHECK_ARG(batch <= 65535, SEMIPD_ESHAPE, "min_gru: at most 65535 requests per launch");
   MinGruArgs a{proj, ld, z_off, x_off, g_off, bias_z, bias_x, y, y_ld, state, state_ld, state_indices, seq_lens, q_start, q_len,
                batch, num_tokens, width, out_scale, workspace, 0};
-  const unsigned cb = (unsigned)((width + 255) / 256);
+  // four adjacent channels per thread (one 8- or 16-byte access per row and operand) where every range starts on such a piece
+  const int64_t esz = dtype == SEMIPD_F32 ? 4 : 2;
+  auto piece = [&](const void* ptr, int64_t stride) { return (reinterpret_cast<uintptr_t>(ptr) % (4 * esz)) == 0 && stride % 4 == 0; };
+  const bool v4 = width % 4 == 0 && z_off % 4 == 0 && x_off % 4 == 0 && g_off % 4 == 0 && piece(proj, ld) && piece(y, y_ld) &&
+                  (reinterpret_cast<uintptr_t>(state) % 16) == 0 && state_ld % 4 == 0;
+  const unsigned cb = (unsigned)((width / (v4 ? 4 : 1) + 255) / 256);
+  const unsigned cb1 = (unsigned)((width + 255) / 256);
   // long portions in chunks: from a few chunks per request up the three passes beat one thread walking every row
   const bool chunked = q_start != nullptr && max_q_len > 4 * kChunk && workspace != nullptr;
   if (!chunked) {
-    SEMIPD_DISPATCH_DTYPE(dtype, T, hipLaunchKernelGGL((min_gru_rows_kernel<T>), dim3(cb, (unsigned)batch), dim3(256), 0,
-                                                       as_stream(stream), a));
+    SEMIPD_DISPATCH_DTYPE(dtype, T, {
+      if (v4) hipLaunchKernelGGL((min_gru_rows_kernel<T, 4>), dim3(cb, (unsigned)batch), dim3(256), 0, as_stream(stream), a);
+      else hipLaunchKernelGGL((min_gru_rows_kernel<T, 1>), dim3(cb, (unsigned)batch), dim3(256), 0, as_stream(stream), a);
+    });
     return launch_status("min_gru");
   }
   a.n_chunks = (num_tokens + kChunk - 1) / kChunk + batch;
   SEMIPD_CHECK_ARG(workspace_bytes >= a.n_chunks * 2 * (int64_t)width * 4, SEMIPD_EINVAL, "min_gru: workspace too small");
   SEMIPD_CHECK_ARG(a.n_chunks <= 65535, SEMIPD_ESHAPE, "min_gru: too many chunks for one launch");
   SEMIPD_DISPATCH_DTYPE(dtype, T, {
-    hipLaunchKernelGGL((min_gru_chunk_kernel<T, false>), dim3(cb, (unsigned)a.n_chunks), dim3(256), 0, as_stream(stream), a);
-    hipLaunchKernelGGL(min_gru_chain_kernel, dim3(cb, (unsigned)batch), dim3(256), 0, as_stream(stream), a);
-    hipLaunchKernelGGL((min_gru_chunk_kernel<T, true>), dim3(cb, (unsigned)a.n_chunks), dim3(256), 0, as_stream(stream), a);
+    if (v4) hipLaunchKernelGGL((min_gru_chunk_kernel<T, 4, false>), dim3(cb, (unsigned)a.n_chunks), dim3(256), 0, as_stream(stream), a);
+    else hipLaunchKernelGGL((min_gru_chunk_kernel<T, 1, false>), dim3(cb, (unsigned)a.n_chunks), dim3(256), 0, as_stream(stream), a);
+    hipLaunchKernelGGL(min_gru_chain_kernel, dim3(cb1, (unsigned)batch), dim3(256), 0, as_stream(stream), a);
+    if (v4) hipLaunchKernelGGL((min_gru_chunk_kernel<T, 4, true>), dim3(cb, (unsigned)a.n_chunks), dim3(256), 0, as_stream(stream), a);
+    else hipLaunchKernelGGL((min_gru_chunk_kernel<T, 1, true>), dim3(cb, (unsigned)a.n_chunks), dim3(256), 0, as_stream(stream), a);
   });
   return launch_status("min_gru(chunked)");
 }

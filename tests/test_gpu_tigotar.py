@@ -56,7 +56,7 @@ def test_dyn_tanh_seam(dtype, rows, width):
 
 # ----------------------------------------------------------------------------------------------- bias + rotation + value norm + store
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,G,D,E,rot", [(4, 2, 32, 16, 32), (3, 1, 20, 12, 10), (2, 2, 64, 256, 2), (1, 1, 128, 100, 0), (2, 1, 8, 500, 4),
+@pytest.mark.parametrize("H,G,D,E,rot", [(4, 2, 32, 16, 32), (3, 1, 20, 12, 10), (2, 2, 64, 256, 2), (1, 1, 128, 100, 0), (2, 1, 8, 500, 4), (6, 2, 96, 160, 96), (2, 2, 64, 64, 16),
                                          (5, 5, 160, 8, 96)])
 def test_bias_rotation_value_norm_store(dtype, H, G, D, E, rot):
     from semi_pd_amd import ops
