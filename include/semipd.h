@@ -865,6 +865,10 @@ int semipd_min_gru(const void* proj, int64_t ld, int64_t z_off, int64_t x_off, i
                    int64_t batch, int64_t num_tokens, int64_t max_q_len, int width, float out_scale, float* workspace,
                    int64_t workspace_bytes, int dtype, void* stream);
 int64_t semipd_min_gru_workspace(int64_t num_tokens, int64_t batch, int width);
+/* Router logits of a small batch in fp32: out[t, e] = sum_i hidden[t, i] * weight[e, i]; hidden rows of `dtype` (row
+ * stride ld), weight fp32 [num_experts, width], out fp32 [num_tokens, num_experts].  No reference counterpart. */
+int semipd_router_logits(const void* hidden, int64_t ld, const float* weight, float* out, int64_t num_tokens, int width,
+                         int num_experts, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -188,6 +188,8 @@ __global__ void __launch_bounds__(256) bias_rope_vnorm_kv_store_kernel(
 // computed once (into LDS) and serve every q and k head; a head of q / k is D / 8 pieces of four pairs, taken by the lanes in
 // turn; value heads go Lp lanes each (the power of two above E / 8) with the sum of squares reduced inside the group.
 // D, E, rot multiples of 8 (a piece is rotated wholly or not at all), rot <= 512, E <= 512.
+// gridDim.y waves share a token (few tokens: a decode batch would otherwise be a handful of waves walking all heads in turn);
+// each computes the angles it needs itself.
 template <typename T>
 __global__ void __launch_bounds__(256) bias_rope_vnorm_kv_store_vec_kernel(
     T* __restrict__ qkv, int64_t ld, int64_t num_tokens, int H, int G, int D, int E, int64_t k_off, int64_t v_off,
@@ -211,7 +213,8 @@ __global__ void __launch_bounds__(256) bias_rope_vnorm_kv_store_vec_kernel(
   T* row = qkv + t * ld;
   const int64_t slot = loc[t];
   const int L = D >> 3, n_qk = (H + G) * L;
-  for (int idx = lane; idx < n_qk; idx += 64) {
+  const int part = blockIdx.y, parts = gridDim.y;
+  for (int idx = lane + 64 * part; idx < n_qk; idx += 64 * parts) {
     const int h = idx / L, pc = idx - h * L;
     const bool is_q = h < H;
     const int hh = is_q ? h : h - H;
@@ -246,7 +249,7 @@ __global__ void __launch_bounds__(256) bias_rope_vnorm_kv_store_vec_kernel(
   int Lp = 1;
   while (Lp < LV) Lp <<= 1;
   const int per_iter = 64 / Lp, sl = lane & (Lp - 1);
-  for (int g0 = 0; g0 < G; g0 += per_iter) {
+  for (int g0 = per_iter * part; g0 < G; g0 += per_iter * parts) {
     const int g = g0 + lane / Lp;
     const bool on = g < G && sl < LV;
     float f[8], ss = 0.f;
@@ -1072,8 +1075,12 @@ extern "C" int semipd_bias_rope_vnorm_kv_store(void* qkv, int64_t ld, int64_t nu
       ld % 8 == 0 && k_off % 8 == 0 && v_off % 8 == 0 && aligned16(qkv) && aligned16(k_pool) && aligned16(v_pool) &&
       (!bias_q || aligned16(bias_q)) && (!bias_k || aligned16(bias_k)) && (!bias_v || aligned16(bias_v))) {
     const unsigned vb = (unsigned)((num_tokens + 3) / 4);
+    // about a thousand waves at least: the waves of a token split its heads' pieces
+    const int64_t iters = ((int64_t)(num_q_heads + num_kv_heads) * (qk_dim / 8) + 63) / 64;
+    int64_t parts = 1024 / (num_tokens < 1024 ? num_tokens : 1024);
+    parts = parts < 1 ? 1 : (parts > iters ? iters : parts);
     SEMIPD_DISPATCH_HALF(dtype, T,
-                         hipLaunchKernelGGL((bias_rope_vnorm_kv_store_vec_kernel<T>), dim3(vb), dim3(256), 0, as_stream(stream),
+                         hipLaunchKernelGGL((bias_rope_vnorm_kv_store_vec_kernel<T>), dim3(vb, (unsigned)parts), dim3(256), 0, as_stream(stream),
                                             (T*)qkv, ld, num_tokens, num_q_heads, num_kv_heads, qk_dim, v_dim, k_off, v_off,
                                             (const T*)bias_q, (const T*)bias_k, (const T*)bias_v, positions, inv_freq, rot_dims,
                                             eps, (T*)k_pool, (T*)v_pool, loc));

@@ -529,11 +529,60 @@ template <typename T>
 int launch_moe_tiled_gemm_silu(T* c, const T* a, const T* w, const int32_t* sorted_ids, const int32_t* expert_ids,
                                const int32_t* num_post_pad, int64_t num_valid, int64_t n, int64_t k, int64_t max_sorted,
                                int top_k_div, hipStream_t st);
+
+// Router logits of a small batch in fp32: out[t, e] = sum_i h[t, i] * w[e, i], h rows of the activation type, w fp32.  A
+// workgroup per token, its four waves take the experts in turn, a lane 8 consecutive elements per step (VEC) or one.  For
+// decode batches: the library's fp32 GEMM at 32 x 8 x 4096 takes three times as long, and wants the rows converted first.
+template <typename T, bool VEC>
+__global__ void __launch_bounds__(256) router_logits_kernel(const T* __restrict__ h, int64_t ld, const float* __restrict__ w,
+                                                            float* __restrict__ out, int W, int X) {
+  const int64_t t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const T* row = h + t * ld;
+  for (int e = wave; e < X; e += 4) {
+    const float* we = w + (int64_t)e * W;
+    float acc = 0.f;
+    if constexpr (VEC) {
+      for (int i = lane * 8; i < W; i += 64 * 8) {
+        float x[8];
+        if constexpr (sizeof(T) == 2) {
+          const Vec16<T> v = load16(row + i);
+#pragma unroll
+          for (int u = 0; u < 8; ++u) x[u] = Elem<T>::to_f(v.e[u]);
+        } else {
+#pragma unroll
+          for (int u = 0; u < 8; ++u) x[u] = Elem<T>::to_f(row[i + u]);
+        }
+        const float4 a = *reinterpret_cast<const float4*>(we + i), b = *reinterpret_cast<const float4*>(we + i + 4);
+        acc += x[0] * a.x + x[1] * a.y + x[2] * a.z + x[3] * a.w + x[4] * b.x + x[5] * b.y + x[6] * b.z + x[7] * b.w;
+      }
+    } else {
+      for (int i = lane; i < W; i += 64) acc += Elem<T>::to_f(row[i]) * we[i];
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) out[t * X + e] = acc;
+  }
+}
+
 }  // namespace semipd
 
 using namespace semipd;
 
 extern "C" {
+
+int semipd_router_logits(const void* hidden, int64_t ld, const float* weight, float* out, int64_t num_tokens, int width,
+                         int num_experts, int dtype, void* stream) {
+  SEMIPD_CHECK_ARG(num_tokens >= 0 && width > 0 && num_experts > 0 && ld >= width, SEMIPD_EINVAL, "router_logits: bad sizes");
+  if (num_tokens == 0) return 0;
+  SEMIPD_CHECK_ARG(hidden && weight && out, SEMIPD_EINVAL, "router_logits: null pointer");
+  const int64_t esz = dtype == SEMIPD_F32 ? 4 : 2;
+  const bool vec = width % 8 == 0 && aligned16(hidden) && (ld * esz) % 16 == 0 && aligned16(weight);
+  SEMIPD_DISPATCH_DTYPE(dtype, T, {
+    if (vec) hipLaunchKernelGGL((router_logits_kernel<T, true>), dim3((unsigned)num_tokens), dim3(256), 0, as_stream(stream), (const T*)hidden, ld, weight, out, width, num_experts);
+    else hipLaunchKernelGGL((router_logits_kernel<T, false>), dim3((unsigned)num_tokens), dim3(256), 0, as_stream(stream), (const T*)hidden, ld, weight, out, width, num_experts);
+  });
+  return launch_status("router_logits");
+}
 
 int semipd_topk_softmax(const void* gating, float* topk_weights, int32_t* topk_ids,
                         int64_t num_tokens, int num_experts, int topk, int renormalize, int dtype,

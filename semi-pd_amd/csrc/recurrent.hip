@@ -35,7 +35,7 @@ struct MinGruArgs {
   int64_t n_chunks;                   // an upper bound (chunks past the last request's do nothing)
 };
 
-constexpr int kChunk = 64;
+constexpr int kChunk = 32;
 
 // 1 / (1 + exp(-x)) from one v_exp_f32 and one v_rcp_f32 (overflow of the exponential gives 0)
 __device__ __forceinline__ float sigmoidf_(float x) {
@@ -162,7 +162,7 @@ __global__ void __launch_bounds__(256) min_gru_chunk_kernel(MinGruArgs a) {
     S[j] = WRITE ? wk[a.R + c + j] : 0.f;
     A[j] = 1.0f;
   }
-#pragma unroll 4
+#pragma unroll 8
   for (int64_t i = i0; i < i1; ++i) {
     const T* row = (const T*)a.p + (t0 + i) * a.ld;
     gru_step<T, V>(row, a, c, bz, bx, S, keep);
@@ -235,7 +235,7 @@ extern "C" int semipd_min_gru(const void* proj, int64_t ld, int64_t z_off, int64
   const unsigned cb = (unsigned)((width / (v4 ? 4 : 1) + 255) / 256);
   const unsigned cb1 = (unsigned)((width + 255) / 256);
   // long portions in chunks: from a few chunks per request up the three passes beat one thread walking every row
-  const bool chunked = q_start != nullptr && max_q_len > 4 * kChunk && workspace != nullptr;
+  const bool chunked = q_start != nullptr && max_q_len > 8 * kChunk && workspace != nullptr;
   if (!chunked) {
     SEMIPD_DISPATCH_DTYPE(dtype, T, {
       if (v4) hipLaunchKernelGGL((min_gru_rows_kernel<T, 4>), dim3(cb, (unsigned)batch), dim3(256), 0, as_stream(stream), a);

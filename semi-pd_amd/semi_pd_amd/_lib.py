@@ -162,6 +162,7 @@ _SIGNATURES = {
     "semipd_min_gru": [_vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32,
                        _f32, _vp, _i64, _i32, _vp],
     "semipd_min_gru_workspace": [_i64, _i64, _i32],
+    "semipd_router_logits": [_vp, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _vp],
 }
 _RESTYPES = {"semipd_last_error": C.c_char_p, "semipd_lm_head_argmax_workspace": _sz,
              "semipd_linear_workspace": _sz, "semipd_stream_linear_workspace": _sz, "semipd_dense_gemm_report": _sz, "semipd_ar_meta_size": _sz, "semipd_ar_region_size": _sz,

@@ -453,8 +453,7 @@ class UngatedMoE(nn.Module):
             self.w_down_cat = self.w_down.permute(1, 0, 2).reshape(K, E * F).contiguous()
 
     def route(self, hidden_states: torch.Tensor):
-        logits = torch.mm(hidden_states.float(), self.router.t())
-        return ops.topk_softmax(logits, self.top_k, True)
+        return ops.topk_softmax(ops.router_logits(hidden_states, self.router), self.top_k, True)
 
     def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
         topk_weights, topk_ids = self.route(hidden_states)

@@ -1562,3 +1562,21 @@ def window_attention_fwd(q: torch.Tensor, out: torch.Tensor, k_buffer: torch.Ten
                                       ptr(q_start), ptr(q_len), B, T, int(max_q_len), H, G, D, E, float(sm_scale), int(window),
                                       int(keep_first), ptr(head_bias), 1 if sigmoid else 0, ptr(sink), float(out_scale),
                                       int(form), dtype_code(q.dtype), current_stream(q.device)), "window_attention")
+
+
+ROUTER_LOGITS_MAX_ROWS = 256
+
+
+def router_logits(hidden_states: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """fp32 router logits [T, X] = hidden [T, W] (activation type or fp32) x weight [X, W] (fp32), accumulated in fp32: the
+    small-batch kernel of csrc/moe.hip up to ROUTER_LOGITS_MAX_ROWS rows, the library's fp32 GEMM above."""
+    if hidden_states.dim() != 2 or hidden_states.stride(1) != 1 or weight.dtype != torch.float32 or not weight.is_contiguous() \
+            or weight.shape[1] != hidden_states.shape[1]:
+        raise RuntimeError("router_logits: hidden [T, W] with contiguous rows, weight fp32 [X, W] contiguous")
+    T, W = hidden_states.shape
+    if T > ROUTER_LOGITS_MAX_ROWS:
+        return torch.mm(hidden_states.float(), weight.t())
+    out = torch.empty((T, weight.shape[0]), dtype=torch.float32, device=hidden_states.device)
+    check(_lib.load().semipd_router_logits(ptr(hidden_states), hidden_states.stride(0), ptr(weight), ptr(out), T, W, weight.shape[0],
+                                           dtype_code(hidden_states.dtype), current_stream(hidden_states.device)), "router_logits")
+    return out

@@ -301,7 +301,7 @@ def _tigotar_kernel_pairs(s, window, keep, dev):
     t_new = _timed(lambda: ops.min_gru(p, H * D + G * D + G * E, H * D + G * D + G * E + R, H * D + G * D + G * E + 2 * R, R, bb, bb, yb,
                                        state, st4, lens, q_start, q_len, L))
     t_old = _timed(lambda: ops.bias_relu_square_(u, bb))
-    out.append((f"minGRU over {B} x {L} tokens, {R} channels (three passes over chunks of 64; like: an in-place element-wise kernel over as many rows)",
+    out.append((f"minGRU over {B} x {L} tokens, {R} channels (three passes over chunks of 32; like: an in-place element-wise kernel over as many rows)",
                 rec(t_new, nbytes=Tn * R * 2.0 * (3 + 2 + 1)), rec(t_old, nbytes=Tn * R * 2.0 * 2)))
     pd = torch.randn(B2, cols, device=dev, dtype=dt)
     yd = torch.empty(B2, R, device=dev, dtype=dt)
