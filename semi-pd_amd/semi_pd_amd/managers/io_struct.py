@@ -102,6 +102,8 @@ class GetNextPrefillBatchOutput:
     # whole decode step long when the loop is overlapped); the decode instance knows them on the host, so they
     # travel with the reply and the table is only needed for prefix tokens (chunked prefill, re-sent requests).
     extend_slots: Optional[List[List[int]]] = None
+    # models with recurrent layers: each request's row of the (shared) recurrent-state pool, allocated by the decode instance
+    state_slots: Optional[List[int]] = None
 
 
 @dataclass

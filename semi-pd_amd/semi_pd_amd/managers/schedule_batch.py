@@ -101,13 +101,16 @@ class ChunkCache:
             req.state_slot = None
 
     def cache_finished_req(self, req: Req):
-        self.release_state(req)
         # KV exists for every token but the last sampled one; a slot taken for a step that runs beyond the end of
         # the request (overlapped decode loop) stays in req.kv_slots and is released when that step is processed
         n = len(req.origin_input_ids) + len(req.output_ids) - 1
         self.req_to_token_pool.free(req.req_pool_idx)
         self.token_to_kv_pool_allocator.free(req.kv_slots[:n])
         req.kv_slots = req.kv_slots[n:]
+        if not req.kv_slots:
+            # (a step launched beyond the end of the request still updates its recurrent-state row: the row goes back with
+            # that step's slot, where the overlapped decode loop processes it)
+            self.release_state(req)
 
     def cache_unfinished_req(self, req: Req):
         kv_indices = self.req_to_token_pool.req_to_token[req.req_pool_idx, : len(req.fill_ids)]
@@ -216,7 +219,8 @@ class ScheduleBatch:
 
     # ---------------------------------------------------------------------------- extend
     def prepare_for_extend(self, pre_allocated_req_pool_indices: Optional[List[int]] = None,
-                           pre_allocated_slots: Optional[List[List[int]]] = None):
+                           pre_allocated_slots: Optional[List[List[int]]] = None,
+                           pre_allocated_state_slots: Optional[List[int]] = None):
         self.forward_mode = ForwardMode.EXTEND
         bs = len(self.reqs)
         if pre_allocated_req_pool_indices is None:
@@ -238,7 +242,12 @@ class ScheduleBatch:
         table = self.req_to_token_pool.req_to_token
         for r, idx in zip(reqs, req_pool_indices):
             r.req_pool_idx = idx
-        self.alloc_state_slots()
+        if pre_allocated_state_slots is not None:
+            # prefill instance: the rows the decode instance allocated (it alone allocates and releases them)
+            assert len(pre_allocated_state_slots) == bs
+            self.state_indices = host_list_to_device(list(pre_allocated_state_slots), torch.int64, dev)
+        else:
+            self.alloc_state_slots()
         if pre_allocated_req_pool_indices is None:
             # decode instance: the only allocator.  Writes the *shared* table.
             out_cpu = self.alloc_token_slots(extend_num_tokens)

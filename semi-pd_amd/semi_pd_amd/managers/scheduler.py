@@ -63,8 +63,9 @@ class SchedulerBase:
         self.send_to_detokenizer = send_to_detokenizer
         self.req_to_token_pool = model_runner.req_to_token_pool
         self.token_to_kv_pool_allocator = model_runner.token_to_kv_pool_allocator
+        # (the prefill instance maps the decode instance's pools and allocates nothing: state rows come with the reply)
         self.tree_cache = ChunkCache(self.req_to_token_pool, self.token_to_kv_pool_allocator,
-                                     getattr(model_runner, "state_pool", None))
+                                     getattr(model_runner, "state_pool", None) if role != InstanceRole.PREFILL else None)
         self.max_total_num_tokens = model_runner.max_total_num_tokens
         self.max_running_requests = server_args.max_running_requests
         self.max_prefill_tokens = server_args.max_prefill_tokens

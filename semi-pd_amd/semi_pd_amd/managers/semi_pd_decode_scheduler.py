@@ -162,7 +162,8 @@ class SemiPDDecodeScheduler(SchedulerBase):
                 req_pool_indices=[r.req_pool_idx for r in batch.reqs],
                 prefix_lens=prefix_lens,
                 extend_input_lens=[r.extend_input_len for r in batch.reqs],
-                extend_slots=[r.kv_slots[p: p + r.extend_input_len] for r, p in zip(batch.reqs, prefix_lens)]))
+                extend_slots=[r.kv_slots[p: p + r.extend_input_len] for r, p in zip(batch.reqs, prefix_lens)],
+                state_slots=([r.state_slot for r in batch.reqs] if self.tree_cache.state_pool is not None else None)))
 
     def _admit(self, recv_req: GetNextPrefillBatchInput) -> Optional[ScheduleBatch]:
         if self.chunked_req:
@@ -341,6 +342,7 @@ class SemiPDDecodeScheduler(SchedulerBase):
                 # it ended one step earlier and ran once more: drop the token, release the slot of that step
                 alloc.free(req.kv_slots)
                 req.kv_slots = []
+                self.tree_cache.release_state(req)     # (that step still updated the request's recurrent-state row)
                 continue
             req.output_ids.append(int(tok))
             self._record_logprob(req, i, logprobs)

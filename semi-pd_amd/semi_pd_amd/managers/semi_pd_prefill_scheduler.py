@@ -145,7 +145,8 @@ class SemiPDPrefillScheduler(SchedulerBase):
         batch = ScheduleBatch.init_new(can_run_list, self.req_to_token_pool, self.token_to_kv_pool_allocator,
                                        self.tree_cache, self.device)
         batch.prepare_for_extend(pre_allocated_req_pool_indices=resp.req_pool_indices,
-                                 pre_allocated_slots=getattr(resp, "extend_slots", None))
+                                 pre_allocated_slots=getattr(resp, "extend_slots", None),
+                                 pre_allocated_state_slots=getattr(resp, "state_slots", None))
         return batch
 
     def _propose(self) -> bool:

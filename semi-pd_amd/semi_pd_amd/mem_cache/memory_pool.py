@@ -293,9 +293,15 @@ class RecurrentStatePool:
         self.slab: Optional[torch.Tensor] = None
         self.buffers: List[torch.Tensor] = []
         if not bypass_create_buffers:
-            self.slab = ipc_safe_zeros((self.size + 1, self.row_width), torch.float32, device)
-            self.buffers = [self.slab[:, o: o + w] for o, w in zip(self.offsets, self.widths)]
+            self.attach(ipc_safe_zeros((self.size + 1, self.row_width), torch.float32, device))
         self.clear()
+
+    def attach(self, slab: torch.Tensor):
+        """Use `slab` ([size + 1, row_width] fp32) as the pool's memory: its own allocation, or the decode instance's slab
+        mapped into the prefill instance (bypass_create_buffers; the prefill instance never allocates rows)."""
+        assert tuple(slab.shape) == (self.size + 1, self.row_width) and slab.dtype == torch.float32
+        self.slab = slab
+        self.buffers = [slab[:, o: o + w] for o, w in zip(self.offsets, self.widths)]
 
     def clear(self):
         self._free = collections.deque(range(1, self.size + 1))

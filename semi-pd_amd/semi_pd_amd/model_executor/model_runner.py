@@ -330,10 +330,7 @@ class ModelRunner:
         self.state_pool = None
         widths = getattr(self.model, "state_geometry", None)
         if widths:
-            if self.instance_role != InstanceRole.OTHER:
-                raise ValueError("models with recurrent layers run in the unified engine only: the Semi-PD instances share "
-                                 "the KV pools and the request table between processes, not a state pool")
-            self.state_pool = RecurrentStatePool(self.max_running_requests, widths, dev)
+            self.state_pool = RecurrentStatePool(self.max_running_requests, widths, dev, bypass_create_buffers=bypass)
 
     # ------------------------------------------------------------------------------------ IPC export
     @torch.no_grad()
@@ -395,10 +392,16 @@ class ModelRunner:
                        "numel": pool.kv_buffer[0].numel(), "layer_num": pool.layer_num}
         kv_info["max_total_num_tokens"] = self.max_total_num_tokens
         r2t = self.req_to_token_pool.req_to_token
+        state_handle = state_info = None
+        if self.state_pool is not None:
+            slab = self.state_pool.slab
+            state_handle = list(get_ipc_handle(slab))
+            state_info = {"shape": tuple(slab.shape), "dtype": slab.dtype, "numel": slab.numel()}
         return IPCInfo(params_info=params_info, weight_handles=weight_handles,
                        register_buffer_handles=buffer_handles, kv_cache_handles=kv_handles,
                        kvcache_info=kv_info, req_to_token_handle=list(get_ipc_handle(r2t)),
-                       req_to_token_info={"shape": tuple(r2t.shape), "dtype": r2t.dtype, "numel": r2t.numel()})
+                       req_to_token_info={"shape": tuple(r2t.shape), "dtype": r2t.dtype, "numel": r2t.numel()},
+                       state_handle=state_handle, state_info=state_info)
 
     # ------------------------------------------------------------------------------------ IPC import
     def _import(self, handle, info) -> torch.Tensor:
@@ -457,6 +460,12 @@ class ModelRunner:
         ri = ipc_info.req_to_token_info
         self.req_to_token_pool.req_to_token = self._import(
             ipc_info.req_to_token_handle, {"numel": ri["numel"], "dtype": ri["dtype"], "shape": ri["shape"]})
+        if self.state_pool is not None:
+            si = getattr(ipc_info, "state_info", None)
+            if si is None or tuple(si["shape"]) != (self.state_pool.size + 1, self.state_pool.row_width):
+                raise RuntimeError("the decode instance exported no recurrent-state pool of this model's shape")
+            self.state_pool.attach(self._import(ipc_info.state_handle, {"numel": si["numel"], "dtype": si["dtype"],
+                                                                        "shape": si["shape"]}))
 
     # ------------------------------------------------------------------------------------ library GEMM selection
     def tune_dense_gemms(self, rows=(1024, 2048, 128, 256, 512, 1536, 3072, 4096, 6144, 8192), num_full_search: int = 2) -> str:

@@ -14,7 +14,7 @@ import ctypes as C
 import os
 from dataclasses import dataclass
 from enum import Enum
-from typing import Dict, List
+from typing import Dict, List, Optional
 
 import torch
 
@@ -42,6 +42,9 @@ class IPCInfo:
     kvcache_info: dict
     req_to_token_handle: list
     req_to_token_info: dict
+    # models with recurrent layers: the slab of per-request state rows (mem_cache/memory_pool.py: RecurrentStatePool)
+    state_handle: Optional[list] = None
+    state_info: Optional[dict] = None
 
 
 class InstanceRole(Enum):

@@ -347,6 +347,12 @@ CONFIGS = {
     "awkward": {"architecture": "Tigotar", "vocab": 301, "width": 100, "norm": {"eps": 1e-5}, "logit_scale": 2.0,
                 "layers": [_layer(_left(3, 1, 20, 12, 7, 9, 10), 36, 0.9, 1.2, (3, 2, 28)),
                            _layer(_left(2, 2, 24, 20, 1000, 2, 24), 52, 1.0, 0.5, None)]},
+    # a span of two layers run twice, then a layer behind it; the kept positions reach past the window of the last layer
+    "tail": {"architecture": "Tigotar", "vocab": 128, "width": 64, "norm": {"eps": 1e-6}, "logit_scale": 0.25,
+             "loop": {"start": 0, "stop": 2, "times": 2},
+             "layers": [_layer(_left(2, 1, 32, 32, 16, 2, 32), 32, 1.0, 1.0, (2, 1, 64)),
+                        _layer(_left(4, 4, 16, 16, 5, 1, 8), 96, 1.2, 0.9, None),
+                        _layer(_left(8, 2, 32, 16, 12, 20, 32), 64, 0.8, 1.1, (5, 3, 40))]},
 }
 
 
@@ -505,10 +511,11 @@ def test_logits_do_not_depend_on_the_cut_or_the_neighbours(mixed_model):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,vocab", [("minimal", 64), ("awkward", 301)])
+@pytest.mark.parametrize("name,vocab", [("minimal", 64), ("awkward", 301), ("tail", 128)])
 def test_other_sizes(name, vocab, dtype, tmp_path):
     """minimal: heads, groups, experts and windows of one, the whole model one repeated span that runs once.  awkward: sizes
-    that no vector path takes (width 100, heads of 20 / 12, 28-wide experts, a vocabulary of 301), no repeated span at all."""
+    that no vector path takes (width 100, heads of 20 / 12, 28-wide experts, a vocabulary of 301), no repeated span at all.
+    tail: the span is in front and a layer follows it."""
     cfg = CONFIGS[name]
     w = _write_checkpoint(str(tmp_path), cfg, seed=5)
     sched = _scheduler(str(tmp_path), dtype, max_tokens=192)
@@ -561,13 +568,24 @@ def test_greedy_generation_through_the_engine(tmp_path):
     _check_generation(cfg, w, prompts, outs, 24)
 
 
-def test_semi_pd_instances_refuse_a_model_with_recurrent_layers(tmp_path):
-    """The Semi-PD instances share KV pools and the request table between processes, not a state pool: a clear refusal."""
-    from semi_pd_amd.entrypoints.engine import _build_runner
-    from semi_pd_amd.semi_pd.utils import InstanceRole
+def test_greedy_generation_through_the_semi_pd_engine(tmp_path):
+    """The same through a prefill and a decode process on one GPU: the pool regions of every layer run, the slab of recurrent
+    state rows and every parameter reach the prefill process through IPC handles; the decode process hands out the state
+    rows, prompts are cut into 48-token portions in the prefill process (the state row carries the recurrence from portion
+    to portion) and decoded in the other."""
+    from semi_pd_amd.entrypoints.engine import Engine
+    from semi_pd_amd.managers.io_struct import SamplingParams
     from semi_pd_amd.server_args import ServerArgs
-    _write_checkpoint(str(tmp_path), CONFIGS["minimal"], seed=1)
-    sa = ServerArgs(model_path=str(tmp_path), load_format="auto", dtype="bfloat16", context_length=64, max_total_tokens=64,
-                    max_running_requests=2, skip_tokenizer_init=True)
-    with pytest.raises(ValueError, match="recurrent"):
-        _build_runner(sa, 0, 0, InstanceRole.DECODE, 29652, max_total_tokens=64)
+    cfg = CONFIGS["mixed"]
+    w = _write_checkpoint(str(tmp_path), cfg, seed=22)
+    prompts = [_tokens(n, cfg["vocab"], seed=100 + n) for n in (5, 90, 47, 130)]
+    sa = ServerArgs(model_path=str(tmp_path), load_format="auto", dtype="bfloat16", context_length=256, max_total_tokens=2048,
+                    max_running_requests=8, cuda_graph_max_bs=8, chunked_prefill_size=48, skip_tokenizer_init=True,
+                    enable_semi_pd=True, cu_mask_mode="env", prefill_cu_percent=50, decode_cu_percent=50, tune_prefill_gemm=False,
+                    watchdog_timeout=120.0)
+    eng = Engine(sa)
+    try:
+        outs = eng.generate(prompts, SamplingParams(max_new_tokens=16, ignore_eos=True), timeout=300)
+    finally:
+        eng.shutdown()
+    _check_generation(cfg, w, prompts, outs, 16)

@@ -18,7 +18,7 @@ from semi_pd_amd.managers.scheduler import Scheduler
 from semi_pd_amd.managers.semi_pd_decode_scheduler import SemiPDDecodeScheduler
 from semi_pd_amd.managers.semi_pd_prefill_scheduler import SemiPDPrefillScheduler
 from semi_pd_amd.managers.transport import NOTHING
-from semi_pd_amd.mem_cache.memory_pool import ReqToTokenPool, TokenToKVPoolAllocator
+from semi_pd_amd.mem_cache.memory_pool import RecurrentStatePool, ReqToTokenPool, TokenToKVPoolAllocator
 from semi_pd_amd.server_args import ServerArgs
 
 VOCAB = 997
@@ -75,15 +75,58 @@ class FakeWorker:
         return None, torch.tensor(ids, dtype=torch.int32)
 
 
-def make_runner(shared=None, size=4000, max_reqs=32, ctx=512):
+class RecurrentFakeWorker(FakeWorker):
+    """The toy model with a recurrence next to its attention: every request folds its tokens, in order, into one number kept
+    in ITS row of the recurrent-state pool (zero where a sequence starts, whatever the row held), and the next token depends
+    on it -- so a row that is shared, lost, released too early, not carried from portion to portion or not handed to the
+    prefill instance changes the generated ids."""
+
+    def forward_batch_generation(self, mwb):
+        _, ids = super().forward_batch_generation(mwb)
+        rows = self.runner.state_pool.get_state_buffer(0)
+        assert mwb.state_indices is not None and (mwb.state_indices > 0).all(), "a request without a state row"
+        assert len(set(mwb.state_indices.tolist())) == len(mwb.state_indices), "two requests share a state row"
+        new = mwb.extend_seq_lens if mwb.extend_seq_lens is not None else [1] * len(mwb.seq_lens)
+        toks, at, out = mwb.input_ids.tolist(), 0, []
+        for row, n, sl, base in zip(mwb.state_indices.tolist(), new, mwb.seq_lens.tolist(), ids.tolist()):
+            s = 0 if sl == n else int(rows[row, 0])
+            for t in toks[at: at + n]:
+                s = fold(s, t)
+            at += n
+            rows[row, 0] = s
+            out.append((base + s) % VOCAB)
+        return None, torch.tensor(out, dtype=torch.int32)
+
+
+def fold(s, t):
+    return (s * 3 + t + 1) % 1009
+
+
+def expected_recurrent(prompt, n):
+    h, out = list(prompt), []
+    for _ in range(n):
+        s = 0
+        for t in h:
+            s = fold(s, t)
+        out.append((toy_next(h) + s) % VOCAB)
+        h.append(out[-1])
+    return out
+
+
+def make_runner(shared=None, size=4000, max_reqs=32, ctx=512, recurrent=False):
     if shared is None:
         r2t = ReqToTokenPool(max_reqs + 1, ctx + 4, "cpu")
     else:
         r2t = ReqToTokenPool(max_reqs + 1, ctx + 4, "cpu", bypass_create_buffers=True)
         r2t.req_to_token = shared.req_to_token_pool.req_to_token  # the IPC mapping
     alloc = TokenToKVPoolAllocator(size, torch.bfloat16, "cpu", None)
-    return SimpleNamespace(device=torch.device("cpu"), req_to_token_pool=r2t,
-                           token_to_kv_pool_allocator=alloc, max_total_num_tokens=size)
+    runner = SimpleNamespace(device=torch.device("cpu"), req_to_token_pool=r2t,
+                             token_to_kv_pool_allocator=alloc, max_total_num_tokens=size)
+    if recurrent:
+        runner.state_pool = RecurrentStatePool(max_reqs, [1], "cpu", bypass_create_buffers=shared is not None)
+        if shared is not None:
+            runner.state_pool.attach(shared.state_pool.slab)   # the IPC mapping
+    return runner
 
 
 def args(**kw):
@@ -94,9 +137,9 @@ def args(**kw):
 
 
 def run_semi_pd(prompts, max_new, sa, size=4000, force_retract=0, interleave=True, sampling_kw=None,
-                worker_cls=None):
-    d_runner = make_runner(size=size)
-    p_runner = make_runner(shared=d_runner, size=size)
+                worker_cls=None, recurrent=False):
+    d_runner = make_runner(size=size, recurrent=recurrent, max_reqs=sa.max_running_requests)
+    p_runner = make_runner(shared=d_runner, size=size, recurrent=recurrent, max_reqs=sa.max_running_requests)
     kv = torch.zeros(size + 1, dtype=torch.int64)
     d_in, p_in, out = Q(), Q(), Q()
     holder = {}
@@ -105,6 +148,8 @@ def run_semi_pd(prompts, max_new, sa, size=4000, force_retract=0, interleave=Tru
     p = SemiPDPrefillScheduler(sa, p_runner, 0, p_in, d_in, bridge)
     holder["d"] = d
     d.tp_worker, p.tp_worker = (worker_cls or FakeWorker)(d_runner, kv), FakeWorker(p_runner, kv)
+    if recurrent:
+        d.tp_worker, p.tp_worker = RecurrentFakeWorker(d_runner, kv), RecurrentFakeWorker(p_runner, kv)
     if force_retract:
         d.forced_retractions = lambda batch: force_retract if batch.batch_size() > 4 else 0
     got = {}
@@ -133,15 +178,18 @@ def run_semi_pd(prompts, max_new, sa, size=4000, force_retract=0, interleave=Tru
     assert d_runner.req_to_token_pool.available_size() == d_runner.req_to_token_pool.size
     assert p_runner.token_to_kv_pool_allocator.available_size() == size, "the prefill instance allocated KV"
     assert not d.scheduled_prefill_batches and not d.waiting_queue and not p.waiting_queue
+    if recurrent:
+        assert d_runner.state_pool.available_size() == d_runner.state_pool.size, "a state row leaked"
+        assert p_runner.state_pool.available_size() == p_runner.state_pool.size, "the prefill instance allocated a state row"
     return [got[f"r{i}"] for i in range(len(reqs))], d, p
 
 
-def run_unified(prompts, max_new, sa, size=4000):
-    runner = make_runner(size=size)
+def run_unified(prompts, max_new, sa, size=4000, recurrent=False):
+    runner = make_runner(size=size, recurrent=recurrent, max_reqs=sa.max_running_requests)
     kv = torch.zeros(size + 1, dtype=torch.int64)
     inbox, out = Q(), Q()
     s = Scheduler(sa, runner, 0, inbox, out)
-    s.tp_worker = FakeWorker(runner, kv)
+    s.tp_worker = (RecurrentFakeWorker if recurrent else FakeWorker)(runner, kv)
     new_of = max_new if isinstance(max_new, (list, tuple)) else [max_new] * len(prompts)
     for i, pr in enumerate(prompts):
         inbox.send_pyobj(TokenizedGenerateReqInput(f"r{i}", None, list(pr),
@@ -155,6 +203,7 @@ def run_unified(prompts, max_new, sa, size=4000):
             for rid, toks in zip(o.rids, o.output_ids):
                 got.setdefault(rid, []).extend(toks)
     assert runner.token_to_kv_pool_allocator.available_size() == size
+    assert not recurrent or runner.state_pool.available_size() == runner.state_pool.size
     return [got[f"r{i}"] for i in range(len(prompts))]
 
 
@@ -171,6 +220,26 @@ def test_semi_pd_equals_unified_equals_history_rule():
     assert got == want
     assert p.stats["prefill_tokens"] == sum(len(x) for x in prompts)
     assert d.stats["decode_tokens"] == 8 * len(prompts)
+
+
+@pytest.mark.parametrize("overlap", [False, True])
+def test_recurrent_state_rows_travel_between_the_instances(overlap):
+    """A model with a recurrent layer: the decode instance hands out the state rows, the prefill instance fills them through
+    the shared slab -- portion by portion for chunked prompts -- and decoding carries on from them; six rows for fourteen
+    requests, so rows are reused as requests end; retracted requests give their row back and start again from zero.  Both
+    decode loops (in the overlapped one a request that ends runs one step more, which still writes its row)."""
+    prompts = prompts_of([150, 20, 200, 9, 77, 130, 5, 64, 33, 1, 90, 12, 40, 71], seed=5)
+    new = [6, 9, 3, 12, 1, 7, 10, 2, 8, 5, 4, 11, 6, 9]
+    want = [expected_recurrent(p, n) for p, n in zip(prompts, new)]
+    kw = dict(max_running_requests=6, chunked_prefill_size=64)
+    assert run_unified(prompts, new, args(enable_semi_pd=False, **kw), recurrent=True) == want
+    got, d, p = run_semi_pd(prompts, new, args(disable_overlap_schedule=not overlap, **kw), recurrent=True)
+    assert [g[:n] for g, n in zip(got, new)] == want
+    assert p.stats["prefill_batches"] > len(prompts)
+    got, d, p = run_semi_pd(prompts[:8], 12, args(disable_overlap_schedule=not overlap, max_running_requests=8), recurrent=True,
+                            force_retract=2, interleave=False)
+    assert got == [expected_recurrent(x, 12) for x in prompts[:8]]
+    assert p.stats["prefill_tokens"] > sum(len(x) for x in prompts[:8]), "no request was re-prefilled"
 
 
 def test_chunked_prefill_across_p_and_d():

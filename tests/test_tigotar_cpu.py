@@ -156,6 +156,32 @@ def test_state_rows_follow_requests_through_batches():
         ScheduleBatch.init_new([c], r2t, alloc, cache, "cpu").alloc_state_slots()
     cache.release_req(b)
     assert b.state_slot is None and states.available_size() == 1 and alloc.available_size() == 64 - 10
+    # a request that ends while a step beyond its end is in flight (the overlapped decode loop) keeps its state row until
+    # that step's slot is given back: the step still writes the row
+    b2 = Req("b2", [1, 2, 3], sp)
+    b2.fill_ids, b2.extend_input_len = [1, 2, 3], 3
+    ScheduleBatch.init_new([b2], r2t, alloc, cache, "cpu").prepare_for_extend()
+    b2.output_ids = [7]
+    b2.kv_slots.append(int(alloc.alloc(1)[0]))          # the slot of the step launched beyond the end
+    row = b2.state_slot
+    cache.cache_finished_req(b2)
+    assert b2.state_slot == row and len(b2.kv_slots) == 1
+    alloc.free(b2.kv_slots)
+    b2.kv_slots = []
+    cache.release_state(b2)
+    assert b2.state_slot is None and states.available_size() == 1
+    b3 = Req("b3", [4, 5], sp)
+    b3.fill_ids, b3.extend_input_len = [4, 5], 2
+    ScheduleBatch.init_new([b3], r2t, alloc, cache, "cpu").prepare_for_extend()
+    b3.output_ids = [9]
+    cache.cache_finished_req(b3)                          # nothing in flight: the row goes back at once
+    assert b3.state_slot is None and states.available_size() == 1
+    # rows that another instance allocated travel with the batch and are never this side's to release
+    guest = Req("g", [1, 2], sp)
+    guest.fill_ids, guest.extend_input_len = [1, 2], 2
+    gb = ScheduleBatch.init_new([guest], r2t, alloc, ChunkCache(r2t, alloc), "cpu")
+    gb.prepare_for_extend(pre_allocated_req_pool_indices=[2], pre_allocated_slots=[[40, 41]], pre_allocated_state_slots=[2])
+    assert gb.state_indices.tolist() == [2] and guest.state_slot is None
     # a request that has lost its state cannot continue from cached tokens
     a.state_slot = None
     with pytest.raises(RuntimeError, match="given up"):
@@ -198,3 +224,21 @@ def test_plain_model_invariants():
     s = torch.softmax(h @ w["l2.mlp.router"].float().T, -1)
     every = sum(s[:, e: e + 1] * (torch.relu(h @ w[f"l2.mlp.e{e}.up"].float().T) ** 2 @ w[f"l2.mlp.e{e}.down"].float().T) for e in range(5))
     torch.testing.assert_close(P.expert_mixture(h, w, "l2.mlp.", mlp), every, rtol=1e-4, atol=1e-5)
+
+
+def test_command_line_of_a_model_folder(tmp_path):
+    """A Tigotar folder on the command line: the class comes from config.json; float32 is accepted (every kernel of the path
+    takes it); the trace runner wants a device."""
+    import argparse
+    from semi_pd_amd.entrypoints import trace_replay
+    from semi_pd_amd.server_args import ServerArgs, add_cli_args, from_cli_args
+    with open(tmp_path / "config.json", "w") as f:
+        json.dump(CFG, f)
+    ap = argparse.ArgumentParser()
+    add_cli_args(ap)
+    sa = from_cli_args(ap.parse_args(["--model-path", str(tmp_path), "--dtype", "float32", "--skip-tokenizer-init"]))
+    assert type(sa.model_config).__name__ == "TigotarConfig" and sa.torch_dtype == torch.float32 and not sa.enable_semi_pd
+    assert ServerArgs(model_path=str(tmp_path), enable_semi_pd=True, skip_tokenizer_init=True).enable_semi_pd
+    if not torch.cuda.is_available():
+        assert trace_replay.main(["--model", str(tmp_path), "--dtype", "bfloat16", "--out", str(tmp_path / "o"),
+                                  "--max-tokens", "64"]) == 2
