@@ -330,7 +330,8 @@ int semipd_gemm_tall_planes(void* out, float* planes, size_t planes_bytes, const
  * block size block_m in {16, 32, 48, 64} (T tokens route at most T rows to one expert: block_m = 16 ceil(T / 16));
  * max_sorted = entries of sorted_token_ids, a multiple of block_m.  c[id, :] = a[id / top_k_div, :] @ w[expert]^T for
  * id < num_valid, times topk_weights[id] when mul_routed_weight; fuse_silu_mul: w[e] = merged [gate; up], output width
- * n / 2, c = SiLU(gate) * up of the products rounded to dtype.  k % 128 == 0, output width % 16 == 0. */
+ * n / 2, c = SiLU(gate) * up of the products rounded to dtype; fuse_silu_mul == 2: c = max(c, 0)^2 of the products rounded
+ * to dtype (experts without a gate branch; not with mul_routed_weight).  k % 128 == 0, output width % 16 == 0. */
 int semipd_moe_stream_gemm(void* c, const void* a, const void* w, const float* topk_weights, const int32_t* sorted_token_ids,
                            const int32_t* expert_ids, const int32_t* num_tokens_post_pad, int64_t num_valid, int64_t n,
                            int64_t k, int64_t max_sorted, int top_k_div, int mul_routed_weight, int fuse_silu_mul, int block_m,

@@ -41,7 +41,7 @@ __device__ inline uint4 sl_load_nt(const void* p) {  // streamed once: keep it o
   return make_uint4(v[0], v[1], v[2], v[3]);
 }
 
-enum { SL_PLAIN = 0, SL_SILU_MUL = 1 };
+enum { SL_PLAIN = 0, SL_SILU_MUL = 1, SL_RELU2 = 2 };   // SL_RELU2 (grouped form): out = max(out, 0)^2, laid out like SL_PLAIN
 
 // Weights through LDS-DMA.  A fragment-shaped register load (16 rows x 64 B per wave instruction) costs the
 // CU's texture-address path ~80 cycles however it is scheduled: a first version of this file that streamed
@@ -268,7 +268,7 @@ stream_gemm_glds_kernel(T* __restrict__ out, float* __restrict__ planes, const T
       }
     return;
   }
-  if (EPI == SL_PLAIN) {
+  if (EPI != SL_SILU_MUL) {
 #pragma unroll
     for (int g = 0; g < NG; ++g)
 #pragma unroll
@@ -283,6 +283,14 @@ stream_gemm_glds_kernel(T* __restrict__ out, float* __restrict__ planes, const T
         if (m < M && n < N) {
           sl_f32x4 v = acc[g][t];
           if (GR) v *= scale;
+          if (EPI == SL_RELU2) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              // the unfused path rounds the GEMM output to T before the activation reads it
+              const float q = Elem<T>::to_f(Elem<T>::from_f(v[j]));
+              v[j] = q > 0.f ? q * q : 0.f;
+            }
+          }
           uint2 p;
           p.x = (uint32_t)Elem<T>::from_f(v[0]).v | ((uint32_t)Elem<T>::from_f(v[1]).v << 16);
           p.y = (uint32_t)Elem<T>::from_f(v[2]).v | ((uint32_t)Elem<T>::from_f(v[3]).v << 16);
@@ -627,7 +635,8 @@ int semipd_stream_linear_f32(float* out, const void* x, const void* weight, int6
  * expert_ids from moe_align_block_size with block size block_m in {16, 32, 48, 64} (a decode batch of T tokens routes
  * at most T rows to one expert, so block_m = 16 ceil(T / 16) never splits an expert); max_sorted = entries of
  * sorted_token_ids, a multiple of block_m.  c[id, :] = a[id / top_k_div, :] @ w[expert]^T for id < num_valid, times
- * topk_weights[id] when mul_routed_weight; fuse_silu_mul: w[e] = merged [gate; up] and c = SiLU(gate) * up. */
+ * topk_weights[id] when mul_routed_weight; fuse_silu_mul 1: w[e] = merged [gate; up] and c = SiLU(gate) * up; 2: c = max(c, 0)^2
+ * (experts without a gate branch), with the rounding of the separate activation kernel. */
 int semipd_moe_stream_gemm(void* c, const void* a, const void* w, const float* topk_weights, const int32_t* sorted_token_ids,
                            const int32_t* expert_ids, const int32_t* num_tokens_post_pad, int64_t num_valid, int64_t n,
                            int64_t k, int64_t max_sorted, int top_k_div, int mul_routed_weight, int fuse_silu_mul, int block_m,
@@ -638,16 +647,19 @@ int semipd_moe_stream_gemm(void* c, const void* a, const void* w, const float* t
   SEMIPD_CHECK_ARG(c && a && w && sorted_token_ids && expert_ids && num_tokens_post_pad, SEMIPD_EINVAL,
                    "moe_stream_gemm: null pointer");
   SEMIPD_CHECK_ARG(!mul_routed_weight || topk_weights, SEMIPD_EINVAL, "moe_stream_gemm: topk_weights required");
-  const int64_t n_out = fuse_silu_mul ? n / 2 : n;
+  SEMIPD_CHECK_ARG(fuse_silu_mul >= 0 && fuse_silu_mul <= 2 && !(fuse_silu_mul == 2 && mul_routed_weight), SEMIPD_EINVAL,
+                   "moe_stream_gemm: epilogue 0 (none), 1 (SiLU * mul) or 2 (squared ReLU, not with the routed weight)");
+  const int64_t n_out = fuse_silu_mul == 1 ? n / 2 : n;
   SEMIPD_CHECK_ARG((block_m == 16 || block_m == 32 || block_m == 48 || block_m == 64) && max_sorted % block_m == 0 &&
-                       k % 128 == 0 && n_out % 16 == 0 && (!fuse_silu_mul || n % 2 == 0) && aligned16(a) && aligned16(w) &&
+                       k % 128 == 0 && n_out % 16 == 0 && (fuse_silu_mul != 1 || n % 2 == 0) && aligned16(a) && aligned16(w) &&
                        (reinterpret_cast<uintptr_t>(c) & 7u) == 0 && num_valid < (1 << 30) && n < (1 << 30) && k < (1 << 30),
                    SEMIPD_ESHAPE, "moe_stream_gemm: block_m in {16, 32, 48, 64}, k %% 128, output width %% 16 required");
   SgGroup grp{sorted_token_ids, expert_ids, num_tokens_post_pad, topk_weights, (int)num_valid, top_k_div, mul_routed_weight};
   hipStream_t st = as_stream(stream);
   int rc = 0;
 #define SGG(MTV) \
-  if (fuse_silu_mul) { SEMIPD_DISPATCH_HALF(dtype, T, rc = (sg_launch_grouped<T, MTV, SL_SILU_MUL>((T*)c, (const T*)a, (const T*)w, grp, max_sorted, (int)n, (int)k, k, n_out, st))); } \
+  if (fuse_silu_mul == 1) { SEMIPD_DISPATCH_HALF(dtype, T, rc = (sg_launch_grouped<T, MTV, SL_SILU_MUL>((T*)c, (const T*)a, (const T*)w, grp, max_sorted, (int)n, (int)k, k, n_out, st))); } \
+  else if (fuse_silu_mul == 2) { SEMIPD_DISPATCH_HALF(dtype, T, rc = (sg_launch_grouped<T, MTV, SL_RELU2>((T*)c, (const T*)a, (const T*)w, grp, max_sorted, (int)n, (int)k, k, n_out, st))); } \
   else { SEMIPD_DISPATCH_HALF(dtype, T, rc = (sg_launch_grouped<T, MTV, SL_PLAIN>((T*)c, (const T*)a, (const T*)w, grp, max_sorted, (int)n, (int)k, k, n_out, st))); }
   if (block_m == 16) { SGG(1) } else if (block_m == 32) { SGG(2) } else if (block_m == 48) { SGG(3) } else { SGG(4) }
 #undef SGG

@@ -395,8 +395,12 @@ def fused_experts_ungated(hidden_states: torch.Tensor, w_up: torch.Tensor, w_dow
     c3 = torch.empty((numel, K), dtype=dt, device=dev)
     wts = topk_weights.reshape(-1)
     if small:
-        ops.moe_stream_gemm(hidden_states, w_up, c1, None, sorted_ids, expert_ids, num_post_pad, numel, topk, False, block_m)
-        act(c1)
+        # (the squared ReLU rides in the first GEMM's epilogue with the rounding of the separate kernel: same bits, one launch fewer)
+        fused = activation == "relu2"
+        ops.moe_stream_gemm(hidden_states, w_up, c1, None, sorted_ids, expert_ids, num_post_pad, numel, topk, False, block_m,
+                            fuse_relu_square=fused)
+        if not fused:
+            act(c1)
         ops.moe_stream_gemm(c1, w_down, c3, wts, sorted_ids, expert_ids, num_post_pad, numel, 1, True, block_m)
     elif tall:
         ops.moe_gemm_tall(hidden_states, w_up, c1, None, sorted_ids, expert_ids, num_post_pad, numel, topk, False, False,

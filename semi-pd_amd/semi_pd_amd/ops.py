@@ -1025,10 +1025,11 @@ def moe_stream_gemm_is_supported(a: torch.Tensor, w: torch.Tensor, fuse_silu_mul
 def moe_stream_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, topk_weights: Optional[torch.Tensor],
                     sorted_token_ids: torch.Tensor, expert_ids: torch.Tensor, num_tokens_post_pad: torch.Tensor,
                     num_valid: int, top_k_div: int, mul_routed_weight: bool, block_m: int,
-                    fuse_silu_mul: bool = False) -> None:
+                    fuse_silu_mul: bool = False, fuse_relu_square: bool = False) -> None:
     """invoke_fused_moe_kernel (fused_moe.py:501-612) for decode-sized calls with the LDS-DMA streaming kernel (grouped
     form of csrc/stream_linear.hip): sorted_token_ids / expert_ids from moe_align_block_size with block size block_m
-    (16, 32, 48 or 64).  c[id] = a[id // top_k_div] @ w[expert].T (SiLU(gate) * up of it with fuse_silu_mul)."""
+    (16, 32, 48 or 64).  c[id] = a[id // top_k_div] @ w[expert].T (SiLU(gate) * up of it with fuse_silu_mul; max(., 0)^2 of
+    it with fuse_relu_square, the epilogue of experts without a gate branch)."""
     E, N, K = w.shape
     n_out = N // 2 if fuse_silu_mul else N
     if not moe_stream_gemm_is_supported(a, w, fuse_silu_mul) or c.shape[-1] != n_out or not c.is_contiguous() \
@@ -1038,10 +1039,12 @@ def moe_stream_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, topk_weig
         raise RuntimeError("moe_stream_gemm: int32 routing tensors expected")
     if mul_routed_weight and (topk_weights is None or topk_weights.dtype != torch.float32):
         raise RuntimeError("moe_stream_gemm: fp32 topk_weights required")
+    if fuse_relu_square and (fuse_silu_mul or mul_routed_weight):
+        raise RuntimeError("moe_stream_gemm: the squared-ReLU epilogue stands alone")
     check(_lib.load().semipd_moe_stream_gemm(ptr(c), ptr(a), ptr(w), ptr(topk_weights), ptr(sorted_token_ids),
                                              ptr(expert_ids), ptr(num_tokens_post_pad), num_valid, N, K,
                                              sorted_token_ids.numel(), top_k_div, int(mul_routed_weight),
-                                             int(fuse_silu_mul), int(block_m), dtype_code(a.dtype),
+                                             2 if fuse_relu_square else int(fuse_silu_mul), int(block_m), dtype_code(a.dtype),
                                              current_stream(a.device)), "moe_stream_gemm")
 
 

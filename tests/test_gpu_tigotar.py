@@ -321,6 +321,30 @@ def test_ungated_experts(dtype, side_by_side, X, K, W, F, T, monkeypatch):
     assert bad <= T // 200, f"{bad} of {T} rows differ"
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T", [1, 19, 64])
+def test_squared_relu_in_the_first_expert_gemm_keeps_the_bits(dtype, T):
+    """Decode-sized calls: the activation in the epilogue of the grouped streaming GEMM against GEMM + the separate kernel."""
+    from semi_pd_amd import ops
+    g = torch.Generator().manual_seed(T)
+    X, K, W, F = 6, 2, 256, 128
+    h = torch.randn(T, W, generator=g).to(dtype).to(DEV)
+    w_up = (torch.randn(X, F, W, generator=g) / W ** 0.5).to(dtype).to(DEV)
+    _, ids = ops.topk_softmax(torch.randn(T, X, generator=g).to(DEV), K, True)
+    block_m = min(64, 16 * -(-T // 16))
+    numel = T * K
+    max_sorted = -(-(numel + X * (block_m - 1)) // block_m) * block_m
+    sorted_ids = torch.empty(max_sorted, dtype=torch.int32, device=DEV)
+    expert_ids = torch.empty(max_sorted // block_m, dtype=torch.int32, device=DEV)
+    post = torch.empty(1, dtype=torch.int32, device=DEV)
+    ops.moe_align_block_size(ids, X, block_m, sorted_ids, expert_ids, post, None, torch.empty(X + 1, dtype=torch.int32, device=DEV))
+    plain, fused = (torch.zeros(numel, F, dtype=dtype, device=DEV) for _ in range(2))
+    ops.moe_stream_gemm(h, w_up, plain, None, sorted_ids, expert_ids, post, numel, K, False, block_m)
+    ops.bias_relu_square_(plain, None)
+    ops.moe_stream_gemm(h, w_up, fused, None, sorted_ids, expert_ids, post, numel, K, False, block_m, fuse_relu_square=True)
+    assert torch.equal(plain, fused) and plain.abs().max() > 0
+
+
 # ----------------------------------------------------------------------------------------------- model level
 def _left(heads, kv_heads, dim, vdim, size, keep, rot):
     return {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": 0.7 * dim ** -0.5,
