@@ -171,4 +171,36 @@ elif which == "fp8mm":
         junk.fill_(1)  # 256 MB: evicts the weights from the Infinity Cache between launches
         ops.w8a8_block_fp8_matmul(xq, wq, xs, ws, [128, 128], torch.bfloat16)
     print("algorithmic_bytes_per_launch", N * K + ws.numel() * 4 + M * K + xs.numel() * 4 + M * N * 2)
+elif which == "tigotar":
+    # the element-wise kernels of a Tigotar layer run at the 8B-sized shape, a prompt batch of 4 x 2048 tokens: the recurrence
+    # (three passes over chunks), the seam between two sublayers, the q / k / v preparation.  Operands alternate between three
+    # sets so that a launch does not find its rows in the Infinity Cache.
+    H, G, D, E, W, R, B, L = 32, 8, 128, 128, 4096, 4096, 4, 2048
+    T = B * L
+    cols = H * D + G * D + G * E + 3 * R
+    dt = torch.bfloat16
+    sets = [(torch.randn(T, cols, device=dev, dtype=dt), torch.randn(T, W, device=dev, dtype=dt), torch.randn(T, W, device=dev))
+            for _ in range(3)]
+    yb = torch.empty(T, R, device=dev, dtype=dt)
+    state = torch.zeros(B + 1, R, device=dev)
+    bb = torch.zeros(R, device=dev, dtype=dt)
+    slots = torch.arange(1, B + 1, device=dev)
+    lens = torch.full((B,), L, device=dev, dtype=torch.int64)
+    q_start = torch.arange(B, device=dev, dtype=torch.int32) * L
+    q_len = torch.full((B,), L, device=dev, dtype=torch.int32)
+    w1, b1, al = torch.ones(W, device=dev, dtype=dt), torch.zeros(W, device=dev, dtype=dt), torch.tensor(0.5, device=dev, dtype=dt)
+    kp = torch.zeros(T + 1, G, D, device=dev, dtype=dt)
+    vp = torch.zeros(T + 1, G, E, device=dev, dtype=dt)
+    loc = torch.arange(1, T + 1, device=dev)
+    pos = torch.arange(T, device=dev) % L
+    bq, bk, bv = (torch.zeros(n, device=dev, dtype=dt) for n in (H * D, G * D, G * E))
+    inv_freq = 10000.0 ** (-2.0 * torch.arange(D // 2, dtype=torch.float32, device=dev) / D)
+    z_off = H * D + G * D + G * E
+    for i in range(9):
+        p, y, res = sets[i % 3]
+        ops.min_gru(p, z_off, z_off + R, z_off + 2 * R, R, bb, bb, yb, state, slots, lens, q_start, q_len, L)
+        ops.dyn_tanh(y, (w1, b1, al), residual=res, params_out=(w1, b1, al))
+        ops.bias_rope_vnorm_kv_store(p, H, G, D, E, H * D, H * D + G * D, bq, bk, bv, pos, inv_freq, D, 1e-6, kp, vp, loc)
+    print("algorithmic_bytes_per_launch min_gru", T * R * 2 * 4, "dyn_tanh", T * W * 12, "bias_rope_vnorm_kv_store",
+          T * 2 * (2 * H * D + 2 * G * D + 2 * G * E))
 torch.cuda.synchronize()
