@@ -33,7 +33,7 @@ from semi_pd_amd import ops
 from semi_pd_amd.distributed import get_tensor_model_parallel_world_size
 from semi_pd_amd.layers.attention_backend import RadixAttention
 from semi_pd_amd.layers.basic import (DynTanh, LogitsProcessor, MergedColumnParallelLinear, ParallelLMHead,
-                                      RowParallelLinear, VocabParallelEmbedding, dense_linear)
+                                      RowParallelLinear, VocabParallelEmbedding)
 from semi_pd_amd.layers.moe import UngatedMoE
 
 
